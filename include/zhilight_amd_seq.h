@@ -74,16 +74,24 @@ int zls_polynorm(const float* z, const float* coef /* host, 4 */, float eps, int
  * proj fp32 (n_tok, ld); weight fp32 (rank); cache (pages, page_size, rank) in `dtype`. */
 int zls_latent_store(const float* proj, int64_t ld, int64_t col0, const float* weight, float eps, int64_t rank, const zls_batch_t* b,
                      void* cache, int dtype, zl_stream_t s);
+/* The same with a rotated key part: the down-projection holds rank + rot numbers from col0; the first rank are normed as above, the last
+ * rot (one key part shared by all heads) are turned by the token's position -- pair (2i, 2i + 1) when interleaved, else (i, i + rot / 2),
+ * by the angle p * freq[i] (freq fp32 (rot / 2)) -- and stored behind the latent: cache rows hold rank + rot numbers.  The last rot of the
+ * qdim coordinates of each of the `heads` query heads (proj[t] from q_col0) are turned the same way in place. */
+int zls_latent_rope_store(float* proj, int64_t ld, int64_t col0, const float* weight, float eps, int64_t rank, int64_t rot, const float* freq,
+                          int interleaved, int64_t q_col0, int64_t heads, int64_t qdim, const zls_batch_t* b, void* cache, int dtype,
+                          zl_stream_t s);
 
 /* Causal attention of every token over its sequence's cached latents c_0 .. c_p, heads sharing the latent:
  *   score_j = scale * (W_uk,h^T q_h) . c_j;  w_j = exp(score_j) / (sum_i exp(score_i) + exp(sink_h));  o_h = W_uv,h (sum_j w_j c_j)
  *   out[t][h] = o_h * sigmoid(gate[t][h])         (sink NULL: no sink term; gate NULL: no gate)
  * q fp32 (n_tok, ldq) from column q_col0, heads x dim; gate fp32 (n_tok, ldg) from column g_col0, one number per head;
  * w_uk (heads * dim, rank), w_uv (heads * vdim, rank) in `dtype`; out (n_tok, heads * vdim) in `dtype`.  fp32 scores, weights and sums. */
+/* window > 0: a token at position p attends to the keys p - window < j <= p only (0: every j <= p). */
 int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0, const float* gate, int64_t ldg, int64_t g_col0, const void* w_uk,
                          const void* w_uv, const float* sink, const void* cache, const zls_batch_t* b, float scale, int64_t heads,
                          int64_t dim, int64_t vdim, int64_t rank, void* out, int dtype, int single_only, void* workspace, int64_t n_splits,
-                         int no_mfma, zl_stream_t s);
+                         int no_mfma, int64_t window, zl_stream_t s);
 int64_t zls_latent_attention_workspace_bytes(int64_t n_tok, int64_t heads, int64_t rank, int64_t n_splits);
 /* The keys of every token are split over n_splits workgroups (the caller picks it so that the launch fills the chip; any value >= 1 is
  * valid) whose partial results go through `workspace`; rank <= 1024.  In bf16 with rank % 8 == 0 and rank <= 512 the split pass runs
@@ -94,9 +102,12 @@ int64_t zls_latent_attention_workspace_bytes(int64_t n_tok, int64_t heads, int64
  * up-projected for the step: k (n_ctx, ldk >= heads * dim) and vt = V^T (heads * vdim, ldv) in bf16, where sequence i's context rows
  * 0 .. pos0 + count - 1 stand at rows / columns ctx_start[i] ..; ctx_start[i] is a multiple of 64 (the rows up to the next multiple of 64
  * exist and hold finite numbers), or -1 for a sequence this call leaves out.  dim, vdim <= 256; ldv % 8 == 0. */
+/* window as above; ctx_pos0 (int32 (n_seq), nullable: zeros): the position of the first row of a sequence's block in k / vt -- a
+ * windowed step need not up-project the context before its oldest visible key. */
 int zls_latent_attention_prompt(const float* q, int64_t ldq, int64_t q_col0, const float* gate, int64_t ldg, int64_t g_col0, const void* k,
                                 int64_t ldk, const void* vt, int64_t ldv, const float* sink, const int32_t* ctx_start, const zls_batch_t* b,
-                                float scale, int64_t heads, int64_t dim, int64_t vdim, void* out, int dtype, zl_stream_t s);
+                                float scale, int64_t heads, int64_t dim, int64_t vdim, void* out, int dtype,
+                                int64_t window, const int32_t* ctx_pos0, zl_stream_t s);
 
 /* ---- state-space (Mamba-2) mixer ---------------------------------------------------------------------------------------------- */
 /* Causal per-channel convolution + SiLU over the columns col0 .. col0 + channels - 1 of proj: out[t][c] = silu(bias[c] + sum_k
@@ -107,6 +118,13 @@ int zls_conv_silu(const float* proj, int64_t ld, int64_t col0, const float* w, c
                   int64_t taps, const zls_batch_t* b, float* out, zl_stream_t s);
 int zls_conv_tail_update(const float* proj, int64_t ld, int64_t col0, float* tail, int64_t channels, int64_t taps, const zls_batch_t* b,
                          zl_stream_t s);
+/* The same convolution with its parts chosen: in_bias (nullable, fp32 (channels)) is added to every input u[t][c] before the taps (inputs
+ * before a sequence's start stay 0; the tail holds inputs with the bias), bias (nullable) after them, act != 0 applies SiLU.
+ * zls_short_conv_tail is its tail update (same in_bias). */
+int zls_short_conv(const float* proj, int64_t ld, int64_t col0, const float* w, const float* bias, const float* in_bias, int act,
+                   const float* tail, int64_t channels, int64_t taps, const zls_batch_t* b, float* out, zl_stream_t s);
+int zls_short_conv_tail(const float* proj, int64_t ld, int64_t col0, const float* in_bias, float* tail, int64_t channels, int64_t taps,
+                        const zls_batch_t* b, zl_stream_t s);
 
 /* The recurrence, one workgroup per (sequence, head), tokens in order:
  *   dt = softplus(dt_raw + dt_bias_h);  S <- exp(-exp(a_log_h) dt) S + dt B x^T;  y = S^T C + d_h x
@@ -126,6 +144,17 @@ int64_t zls_ssm_scan_workspace_bytes(int64_t n_seq, int64_t max_count, int64_t s
  * square.  y fp32 (rows, inner); z = proj[t][z_col0 ..] fp32; weight fp32 (inner); out in `dtype`. */
 int zls_gated_group_norm(const float* y, const float* proj, int64_t ld, int64_t z_col0, const float* weight, float eps, int64_t rows,
                          int64_t inner, int64_t norm_groups, void* out, int dtype, zl_stream_t s);
+
+/* ---- weighted RMS norm ----------------------------------------------------------------------------------------------------------- */
+/* out[i] = x[r] / sqrt(mean(x[r]^2) + eps) * (w + shift), r = rows[i] (rows NULL: r = i); x fp32 (.., width), w fp32 (width), out
+ * (n_rows, width) in `dtype`.  shift = 1 serves weights stored around zero, 0 plain weights. */
+int zls_rms_norm(const float* x, const int32_t* rows, const float* w, float shift, float eps, int64_t n_rows, int64_t width, void* out,
+                 int dtype, zl_stream_t s);
+/* x[t] += y[t] in place (fp32 (rows, width)); with w2 (nullable) also h2[t] = the weighted RMS norm of the new x[t] in `dtype`. */
+int zls_add_rms_norm(float* x, const float* y, float eps, int64_t rows, int64_t width, const float* w2, float shift, void* h2, int dtype,
+                     zl_stream_t s);
+/* z[i] <- cap * tanh(z[i] * scale / cap) for n fp32 numbers in place (cap <= 0: z[i] * scale). */
+int zls_scale_softcap(float* z, int64_t n, float scale, float cap, zl_stream_t s);
 
 /* ---- layer norm --------------------------------------------------------------------------------------------------------------- */
 /* out[i] = (x[r] - mean) / sqrt(var + eps) * w + b with r = rows[i] (rows NULL: r = i), var = mean of the squared deviations; x fp32
@@ -147,40 +176,46 @@ int zls_add_layer_norm(float* x, const float* y, const float* w, const float* b,
  * Queries are written back to proj; keys go to the token's row of k_cache (pages, page_size, kv_heads * dim), values to the token's
  * column of v_cache, whose pages are transposed: (pages, kv_heads * vdim, page_size); both in `dtype`.  k_cache NULL (then v_cache too): only the queries are served -- a layer that reads
  * another layer's cache.  qk_freq fp32 (rot_dims / 2; rot_dims even, <= dim; 0: no rotation), v_freq fp32 (vdim / 2; vdim even).
- * dim, vdim <= 512. */
+ * dim, vdim <= 512.  interleaved != 0: the rotated pairs are the neighbours (2i, 2i + 1) instead of (i, i + rot_dims / 2), pair i turned by
+ * p * qk_freq[i] either way.  vmix_src (nullable, fp32 rows of vmix_ld numbers): the values become (1 - vmix_lambda) v + vmix_lambda *
+ * vmix_src[t][vmix_col0 ..] (kv_heads * vdim numbers of the same token, e.g. an earlier layer's values) before they are cached. */
 int zls_rope_norm_store(float* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, int64_t heads, int64_t kv_heads, int64_t dim,
-                        int64_t vdim, const float* qk_freq, int64_t rot_dims, const float* v_freq, float eps, int qk_norm,
-                        const zls_batch_t* b, void* k_cache, void* v_cache, int dtype, zl_stream_t s);
+                        int64_t vdim, const float* qk_freq, int64_t rot_dims, const float* v_freq, float eps, int qk_norm, int interleaved,
+                        const float* vmix_src, int64_t vmix_ld, int64_t vmix_col0, float vmix_lambda, const zls_batch_t* b, void* k_cache,
+                        void* v_cache, int dtype, zl_stream_t s);
 
-/* Softmax attention of every token over the cached keys j of its sequence with 0 <= p - j < window (window <= 0: all j <= p):
+/* Softmax attention of every token over the cached keys j of its sequence with 0 <= p - j < window (window <= 0: all j <= p), and with
+ * window > 0 also over the kept first keys j < keep_first (j <= p), at their true positions:
  *   w_g(j) = softmax_j(scale * q_g . k_c(g)(j)),  c(g) = g / (heads / kv_heads)
  *   all_kv == 0:  a[g][:]    = sum_j w_g(j) v_c(g)(j)                      nv = vdim numbers per head
  *   all_kv != 0:  a[g][c][:] = sum_j w_g(j) v_c(j) for EVERY kv head c     nv = kv_heads * vdim
  * The second form is what mixing the heads' weights needs (zls_head_mix_gate): sum_j (sum_g T[h][g] w_g(j)) v_c(h)(j) =
  * sum_g T[h][g] a[g][c(h)].  q fp32 (n_tok, ldq) from q_col0 (as zls_rope_norm_store left it).  Scores, weights and sums are fp32.
- * The pages of a token's window are divided over n_splits workgroups (pages_per_split each, from the page of the window's oldest key;
- * n_splits * pages_per_split must cover the longest window of the step); split s leaves acc[t][g][s][:] = sum_j e^(s_j - m) v_j,
+ * The pages of a token's window (after the pages that only hold kept first keys) are divided over n_splits workgroups (pages_per_split
+ * each; n_splits * pages_per_split must cover the longest such list of the step); split s leaves acc[t][g][s][:] = sum_j e^(s_j - m) v_j,
  * unnormalised, and ml[t][g][s] = (m, sum_j e^(s_j - m)); zls_head_mix_gate merges them.  acc fp32 (n_tok, heads, n_splits, nv), ml fp32
  * (n_tok, heads, n_splits, 2).  single_only != 0: only sequences that bring ONE token are served (portions: zls_window_attention_prompt).
  * The value plane holds a page TRANSPOSED, (kv_heads, vdim, page_size), as zls_rope_norm_store writes it.  nv <= 2048, page_size <= 128
  * and a multiple of 8. */
 int zls_window_attention(const float* q, int64_t ldq, int64_t q_col0, const void* k_cache, const void* v_cache, const zls_batch_t* b,
-                         float scale, int64_t window, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim, int all_kv, float* acc,
-                         float* ml, int64_t n_splits, int64_t pages_per_split, int single_only, int dtype, zl_stream_t s);
+                         float scale, int64_t window, int64_t keep_first, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim, int all_kv,
+                         float* acc, float* ml, int64_t n_splits, int64_t pages_per_split, int single_only, int dtype, zl_stream_t s);
 /* The same attention for query TILES on the matrix cores, bf16 only: tile i = tiles[3 i ..] = (first flat token, rows <= 64, sequence
- * index), consecutive tokens of one sequence.  Writes split 0 of acc for its tokens, already normalised, with ml = (0, 1), and
- * ml = (-inf, 0) for the other splits.  page_size 64, dim % 8 == 0, dim <= 256, vdim % 16 == 0. */
+ * index), consecutive tokens of one sequence.  Writes split 0 of acc for its tokens, unnormalised with ml = (m, sum) like the plain
+ * kernel, and ml = (-inf, 0) for the other splits.  page_size 64, dim % 8 == 0, dim <= 256, vdim % 16 == 0. */
 int zls_window_attention_prompt(const float* q, int64_t ldq, int64_t q_col0, const void* k_cache, const void* v_cache, const zls_batch_t* b,
-                                const int32_t* tiles, int64_t n_tiles, float scale, int64_t window, int64_t heads, int64_t kv_heads,
-                                int64_t dim, int64_t vdim, int all_kv, float* acc, float* ml, int64_t n_splits, int dtype, zl_stream_t s);
+                                const int32_t* tiles, int64_t n_tiles, float scale, int64_t window, int64_t keep_first, int64_t heads,
+                                int64_t kv_heads, int64_t dim, int64_t vdim, int all_kv, float* acc, float* ml, int64_t n_splits, int dtype,
+                                zl_stream_t s);
 
 /* out[t][h][:] = turn_back(sum_g talk[h][g] a[t][g][c(h)][:]) * sigmoid(gate[t][h * vdim + :]), a = the splits of acc merged:
- * a[t][g] = sum_s e^(m_s - M) acc[t][g][s] / sum_s e^(m_s - M) l_s.
+ * a[t][g] = sum_s e^(m_s - M) acc[t][g][s] / (sum_s e^(m_s - M) l_s + e^(sink_g - M)), the last term only with sink (fp32 (heads),
+ * nullable: a learned score per head that has no key and no value and is not scaled; M then also covers it).
  * talk fp32 (heads, heads), NULL: no mixing, acc holds vdim numbers per head and split; v_freq (nullable): pair (m, m + vdim / 2) is turned
  * by -p * v_freq[m]; gate fp32 (n_tok, ldg) from g_col0, NULL: no gate; out (n_tok, heads * vdim) in `dtype`. */
 int zls_head_mix_gate(const float* acc, const float* ml, int64_t n_splits, const float* talk, const float* v_freq, const float* gate,
-                      int64_t ldg, int64_t g_col0, const zls_batch_t* b, int64_t heads, int64_t kv_heads, int64_t vdim, void* out, int dtype,
-                      zl_stream_t s);
+                      int64_t ldg, int64_t g_col0, const float* sink, const zls_batch_t* b, int64_t heads, int64_t kv_heads, int64_t vdim, void* out,
+                      int dtype, zl_stream_t s);
 
 /* ---- linear attention with a scalar decay per head and token ---------------------------------------------------------------------- */
 /* S_t = a_t S_{t-1} + b_t k_t v_t^T,  y_t = S_t^T q_t   per head, S fp32 (dim x vdim) carried in state[slot].
@@ -190,9 +225,12 @@ int zls_head_mix_gate(const float* acc, const float* ml, int64_t n_splits, const
  *   one more number per head, n_t . q_t.
  * state fp32 (slots, heads, dim, vdim + norm_col); y fp32 (n_tok, heads * (vdim + norm_col)).  Long portions run in segments exactly as
  * zls_ssm_scan's do (same kernel, workspace from zls_ssm_scan_workspace_bytes(n_seq, max_count, seg_len, heads, vdim + norm_col, dim)). */
+/* decay_v (nullable; then decay_h and decay_t are NULL): fp32 (n_tok, heads * dim), a decay per KEY CHANNEL and token --
+ * S_t = diag(a_t) S_{t-1} + b_t k_t v_t^T (the decay acts on the state's rows). */
 int zls_decay_scan(const float* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, int act, const float* decay_h,
                    const float* decay_t, const float* gain_t, int norm_col, float* state, int64_t heads, int64_t dim, int64_t vdim,
-                   const zls_batch_t* b, float* y, void* workspace, int64_t seg_len, zl_stream_t s);
+                   const zls_batch_t* b, float* y, void* workspace, int64_t seg_len, const float* decay_v,
+                   zl_stream_t s);
 
 /* Exponential gates with a running maximum (per sequence and head, tokens in order; m carried in m_state[slot][h], 0 for a new sequence):
  *   i = cap tanh((zi + i_bias[h]) / cap),  f = log sigmoid(cap tanh((zf + f_bias[h]) / cap))      (cap <= 0: no cap)
@@ -205,17 +243,23 @@ int zls_exp_gates(const float* proj, int64_t ld, int64_t i_col0, int64_t f_col0,
  *   with m_vals (needs norm_col): o = q_scale * o / (max(|q_scale * y[t][h][vdim]|, exp(-m_vals[t][h])) + den_eps);
  *   every one of `norm_groups` equal parts of the row heads * vdim is divided by sqrt(mean(part^2) + eps), times weight (nullable),
  *   times sigmoid(gate[t][g_col0 + c]) (gate nullable).  out (n_tok, heads * vdim) in `dtype`. */
+/* gate_kind 0: the gate is sigmoid(gate); 1: silu(gate).  Without m_vals o is only scaled by q_scale before the norm. */
 int zls_linear_attn_finish(const float* y, int64_t norm_col, float q_scale, const float* m_vals, float den_eps, int64_t heads, int64_t vdim,
                            int64_t norm_groups, const float* weight, float eps, const float* gate, int64_t ldg, int64_t g_col0,
-                           int64_t n_tok, void* out, int dtype, zl_stream_t s);
+                           int64_t n_tok, void* out, int dtype, int gate_kind, zl_stream_t s);
+/* alpha[t][c] = sigmoid(sum_j w2[c][j] u[t][j] + bias[c])^(1 / tau) for c < channels: a decay per channel from `low` numbers per token,
+ * u[t] = proj[t][u_col0 ..] fp32; w2 (channels, low) in `dtype`, bias fp32 (nullable); sums, the log-sigmoid and alpha are fp32. */
+int zls_lowrank_decay(const float* proj, int64_t ld, int64_t u_col0, int64_t low, const void* w2, const float* bias, float tau,
+                      int64_t channels, int64_t n_tok, float* alpha, int dtype, zl_stream_t s);
 
 /* ---- mixture of experts over a ragged step ------------------------------------------------------------------------------------------ */
-/* Router: s = softmax(logits[t]) over all n_out outputs; choice = s + correction (nullable); the outputs form `groups` equal groups of
- * neighbours, a group's score is its largest choice score, only outputs of the `keep` best groups can be chosen (groups <= 1: all);
- * the `top` largest choice scores are chosen (ties: the lower index).  ids int32 (n_tok, top), weights fp32 (n_tok, top) = s of the
- * chosen (scaled by 1 / their sum when renorm != 0).  n_out <= 1024, n_out % groups == 0. */
+/* Router: s = softmax(logits[t]) over all n_out outputs (score_kind 0) or sigmoid(logits[t][i]) of each (score_kind 1); choice = s +
+ * correction (nullable); the outputs form `groups` equal groups of neighbours, a group's score is the sum of its `group_top` largest choice
+ * scores (1: its largest), only outputs of the `keep` best groups can be chosen (groups <= 1: all) -- the others count as minus
+ * infinity; the `top` largest choice scores are chosen (ties: the lower index).  ids int32 (n_tok, top), weights fp32 (n_tok, top) = s of
+ * the chosen (divided by their sum + renorm_eps when renorm != 0).  n_out <= 1024, n_out % groups == 0. */
 int zls_moe_route(const float* logits, int64_t n_tok, int64_t n_out, const float* correction, int64_t groups, int64_t keep, int64_t top,
-                  int renorm, int32_t* ids, float* weights, zl_stream_t s);
+                  int renorm, int score_kind, int64_t group_top, float renorm_eps, int32_t* ids, float* weights, zl_stream_t s);
 /* Sort the n_slots = n_tok * top (token, choice) pairs by expert: pairs whose id is >= n_experts (identity outputs) are left out.
  *   sorted_tok[p] = token of the pair at sorted position p;  slot_pos[t * top + k] = p (or -1);
  *   tiles[3 i ..] = (expert, first position, end position) of the i-th run of at most tile_m positions of one expert, expert = -1 for unused
@@ -233,6 +277,11 @@ int zls_gemm_nt_grouped(const void* x, int64_t ldx, const int32_t* x_rows, const
                         int dtype, int out_dtype, zl_stream_t s);
 /* out[p][c] = silu(gu[p][c]) * gu[p][ff + c]  for rows 0 .. rows - 1 (gu fp32 (rows, 2 ff)), out in `dtype`. */
 int zls_silu_mul(const float* gu, int64_t rows, int64_t ff, void* out, int dtype, zl_stream_t s);
+/* out[p][c] = act(g, u) of gu fp32 (rows, 2 ff) in `dtype`: kind 0 silu(g) u; 1 gelu_tanh(g) u (tanh form); 2 g' sigmoid(alpha g') (u' + 1)
+ * with g' = min(g, limit), u' = clamp(u, -limit, limit).  block 0: g = gu[p][c], u = gu[p][ff + c]; block > 0 (ff % block == 0): the row
+ * holds blocks of `block` gates followed by their `block` ups (the packing of the gated grouped product). */
+int zls_act_mul(const float* gu, int64_t rows, int64_t ff, int kind, float alpha, float limit, int64_t block, void* out, int dtype,
+                zl_stream_t s);
 /* out[t] = sum_k weights[t][k] * (ids[t][k] >= n_experts ? h[t] : y[slot_pos[t * top + k]]), in the order of k; y fp32 (.., width),
  * h (n_tok, width) in `dtype`, out fp32. */
 int zls_moe_combine(const float* y, const int32_t* slot_pos, const int32_t* ids, const float* weights, const void* h, int64_t n_tok,

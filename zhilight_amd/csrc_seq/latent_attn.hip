@@ -1,10 +1,13 @@
 // latent_attn.hip -- attention over a PAGED cache of normed low-rank latents, for every token of a ragged step.
 //
-// Beside csrc/mla_attn.hip (DeepSeek's geometry: 512 + 64 rotated columns, 16-bit, decode rows only, no sink): this one has no rotated
-// part, any rank / head sizes, a learned per-head sink in the softmax denominator, a per-head sigmoid output gate, causal portions of
-// prompts at any offset, and a 32-bit mode.  Only the latent is cached; for single tokens keys and values are never materialised:
+// Beside csrc/mla_attn.hip (DeepSeek's geometry: 512 + 64 rotated columns, 16-bit, decode rows only, no sink): any rank / head sizes, a
+// learned per-head sink in the softmax denominator, a per-head sigmoid output gate, causal portions of prompts at any offset, an optional
+// sliding window, and a 32-bit mode.  Only the latent is cached; for single tokens keys and values are never materialised:
 //     score_j = (W_uk,h^T q_h) . c_j * scale          o_h = W_uv,h . (sum_j w_j c_j)
-// k_latent_store        RMS norm (plain weight) of the down-projection -> the token's cache row
+// A rotated key part shared by all heads rides in the same cached row behind the latent: the row is [c | k_rot], the up-projections get
+// identity columns for it (W_uk) or zeros (W_uv) on the host, and every kernel below sees one longer "latent".
+// k_latent_store        RMS norm (plain weight) of the down-projection -> the token's cache row; the rotated key part behind it and the
+//                       queries' rotated parts (in place), turned by the token's position
 // k_latent_absorb       the query folded through W_uk (and the scale), once per token and head
 // k_latent_split        single tokens (and, in 32-bit serving, every token): the keys split over workgroups, fp32 VALU
 // k_latent_decode_mfma  the same split pass for bf16 on the matrix cores
@@ -14,21 +17,38 @@
 
 namespace {
 
+// rot > 0: the down-projection has rot more columns behind the latent, one rotated key part for all heads: pair (2i, 2i + 1) (interleaved)
+// or (i, i + rot / 2) is turned by pos * freq[i] and stored behind the normed latent (cache rows hold rank + rot numbers); the last rot
+// coordinates of every query head (q_col0, heads x qdim) are turned the same way in place.  A thread owns a whole pair.
 template <int DT>
-__global__ __launch_bounds__(256) void k_latent_store(const float* __restrict__ proj, int64_t ld, int col0, const float* __restrict__ weight,
-                                                      float eps, int rank, const zls_batch_t b, void* __restrict__ cache) {
+__global__ __launch_bounds__(256) void k_latent_store(float* __restrict__ proj, int64_t ld, int col0, const float* __restrict__ weight,
+                                                      float eps, int rank, int rot, const float* __restrict__ freq, int interleaved, int q_col0,
+                                                      int heads, int qdim, const zls_batch_t b, void* __restrict__ cache) {
     __shared__ float red[16];
     const int t = blockIdx.x;
     const int sq = b.tok_seq[t];
     const int pos = b.seq_pos0[sq] + (t - b.seq_start[sq]);
     const int page = b.page_table[(size_t)sq * b.max_pages + pos / b.page_size];
-    const size_t dst = ((size_t)page * b.page_size + pos % b.page_size) * rank;
-    const float* u = proj + (size_t)t * ld + col0;
+    const size_t dst = ((size_t)page * b.page_size + pos % b.page_size) * (rank + rot);
+    float* row = proj + (size_t)t * ld;
+    const float* u = row + col0;
     float ss = 0.f;
     for (int i = threadIdx.x; i < rank; i += 256) ss = fmaf(u[i], u[i], ss);
     ss = zl_block_sum(ss, red);
     const float f = 1.0f / sqrtf(ss / (float)rank + eps);
     for (int i = threadIdx.x; i < rank; i += 256) SeqT<DT>::st(cache, dst + i, u[i] * f * weight[i]);
+    const int half = rot >> 1;
+    for (int w = threadIdx.x; w < (heads + 1) * half; w += 256) {          // vector 0: the key part; 1 ..: the heads' query parts
+        const int vec = w / half, i = w % half;
+        const int a = interleaved ? 2 * i : i, c = interleaved ? 2 * i + 1 : i + half;
+        float sn, cs;
+        seq_sincos((float)pos * freq[i], &sn, &cs);
+        float* src = vec == 0 ? row + col0 + rank : row + q_col0 + (size_t)(vec - 1) * qdim + (qdim - rot);
+        const float x = src[a], y = src[c];
+        const float xr = x * cs - y * sn, yr = y * cs + x * sn;
+        if (vec == 0) { SeqT<DT>::st(cache, dst + rank + a, xr); SeqT<DT>::st(cache, dst + rank + c, yr); }
+        else { src[a] = xr; src[c] = yr; }
+    }
 }
 
 struct AttnP {
@@ -36,6 +56,7 @@ struct AttnP {
     int64_t ldq, ldg;
     int q_col0, g_col0, heads, dim, vdim, rank, single_only, vec;
     float scale;
+    int window;                                    // > 0: a token at position p sees the keys p - window < j <= p only
 };
 
 // Split over keys: workgroup = (token, group of 4 heads, split), a wave per head.  A tile of 16 cached rows is staged once in LDS as fp32
@@ -88,9 +109,10 @@ __global__ __launch_bounds__(256) void k_latent_split(const AttnP p, const zls_b
     const int sq = b.tok_seq[t];
     if (p.single_only && b.seq_start[sq + 1] - b.seq_start[sq] > 1) return;      // portions go to the prompt kernel (workgroup-uniform)
     const int pos = b.seq_pos0[sq] + (t - b.seq_start[sq]);
-    const int nkeys = pos + 1;
+    const int key_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+    const int nkeys = pos + 1 - key_lo;
     const int chunk = ((nkeys + n_splits - 1) / n_splits + 15) & ~15;
-    const int k0 = split * chunk, k1 = min(nkeys, k0 + chunk);
+    const int k0 = key_lo + split * chunk, k1 = min(pos + 1, k0 + chunk);
     const int32_t* pages = b.page_table + (size_t)sq * b.max_pages;
     if (hvalid)
         for (int r = lane; r < p.rank; r += 64) qk[r] = qa[((size_t)t * p.heads + h) * p.rank + r];
@@ -271,7 +293,8 @@ struct FaP {
     int64_t ldq, ldg, ldk, ldv;
     int q_col0, g_col0, heads, dim, vdim, tiles_per_seq, vec_k;
     float scale;
-};
+    int window; const int32_t* ctx_pos0;           // window > 0: keys p - window < j <= p; ctx_pos0 (nullable: 0): the position of a sequence's
+};                                                 // first up-projected row (a windowed step does not bring its whole context)
 
 template <int DK, int DV>
 __global__ __launch_bounds__(256) void k_latent_fa(const FaP p, const zls_batch_t b) {
@@ -283,11 +306,14 @@ __global__ __launch_bounds__(256) void k_latent_fa(const FaP p, const zls_batch_
     const int first = b.seq_start[sq], count = b.seq_start[sq + 1] - first;
     const int cs = p.ctx_start[sq];
     if (cs < 0 || tile * 64 >= count) return;
-    const int pos0 = b.seq_pos0[sq];
+    // positions below are counted from the sequence's first up-projected row (position c0): a key's index there is its row in K / V^T
+    const int c0 = p.ctx_pos0 ? p.ctx_pos0[sq] : 0;
+    const int pos0 = b.seq_pos0[sq] - c0;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nrow = lane & 15, kq = lane >> 4;
     const int qi = tile * 64 + wave * 16 + nrow;
     const bool qvalid = qi < count;
     const int qpos = pos0 + qi;
+    const int j_first = p.window > 0 ? max(0, pos0 + tile * 64 - p.window + 1) & ~63 : 0;     // the tile of the oldest key the first query sees
     const int wave_last = pos0 + min(count, tile * 64 + wave * 16 + 16) - 1;       // the last key any query of this wave sees
     const int block_last = pos0 + min(count, tile * 64 + 64) - 1;
 
@@ -351,8 +377,8 @@ __global__ __launch_bounds__(256) void k_latent_fa(const FaP p, const zls_batch_
             if (idx < DV * 16 * 8) *reinterpret_cast<uint4*>(Vs + (idx >> 3) * VR + (idx & 7) * 8) = vreg[u];
         }
     };
-    fetch_tiles(0);
-    for (int j0 = 0; j0 <= block_last; j0 += 64) {
+    fetch_tiles(j_first);
+    for (int j0 = j_first; j0 <= block_last; j0 += 64) {
         __syncthreads();                                                           // the previous tile is consumed
         publish_tiles();
         __syncthreads();
@@ -373,7 +399,7 @@ __global__ __launch_bounds__(256) void k_latent_fa(const FaP p, const zls_batch_
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int key = j0 + 16 * c + 4 * kq + r;
-                const float v = (qvalid && key <= qpos) ? sc[c][r] * p.scale : -INFINITY;
+                const float v = (qvalid && key <= qpos && (p.window <= 0 || qpos - key < p.window)) ? sc[c][r] * p.scale : -INFINITY;
                 sc[c][r] = v;
                 mx = fmaxf(mx, v);
             }
@@ -453,9 +479,10 @@ __global__ __launch_bounds__(64) void k_latent_decode_mfma(const AttnP p, const 
     const int sq = b.tok_seq[t];
     if (p.single_only && b.seq_start[sq + 1] - b.seq_start[sq] > 1) return;
     const int pos = b.seq_pos0[sq] + (t - b.seq_start[sq]);
-    const int nkeys = pos + 1;
+    const int key_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+    const int nkeys = pos + 1 - key_lo;
     const int chunk = ((nkeys + n_splits - 1) / n_splits + 31) & ~31;
-    const int k0 = split * chunk, k1 = min(nkeys, k0 + chunk);
+    const int k0 = key_lo + split * chunk, k1 = min(pos + 1, k0 + chunk);
     const int32_t* pages = b.page_table + (size_t)sq * b.max_pages;
     const uint16_t* cache = reinterpret_cast<const uint16_t*>(p.cache);
 
@@ -569,14 +596,22 @@ __global__ __launch_bounds__(64) void k_latent_decode_mfma(const AttnP p, const 
 
 }  // namespace
 
-extern "C" int zls_latent_store(const float* proj, int64_t ld, int64_t col0, const float* weight, float eps, int64_t rank, const zls_batch_t* b,
-                                void* cache, int dtype, zl_stream_t s) {
-    ZL_CHECK_ARG(proj && weight && cache && seq_batch_ok(b) && b->page_table && b->page_size > 0 && b->max_pages > 0 && rank > 0, ZL_EINVAL);
-    ZL_CHECK_ARG(col0 >= 0 && col0 + rank <= ld, ZL_ESHAPE);
-#define CALL(DT) hipLaunchKernelGGL((k_latent_store<DT>), dim3(b->n_tok), dim3(256), 0, (hipStream_t)s, proj, ld, (int)col0, weight, eps, (int)rank, *b, cache);
+extern "C" int zls_latent_rope_store(float* proj, int64_t ld, int64_t col0, const float* weight, float eps, int64_t rank, int64_t rot,
+                                     const float* freq, int interleaved, int64_t q_col0, int64_t heads, int64_t qdim, const zls_batch_t* b,
+                                     void* cache, int dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(proj && weight && cache && seq_batch_ok(b) && b->page_table && b->page_size > 0 && b->max_pages > 0 && rank > 0 && rot >= 0, ZL_EINVAL);
+    ZL_CHECK_ARG(col0 >= 0 && col0 + rank + rot <= ld && rot % 2 == 0, ZL_ESHAPE);
+    ZL_CHECK_ARG(rot == 0 || (freq && heads > 0 && qdim >= rot && q_col0 >= 0 && q_col0 + heads * qdim <= ld), ZL_ESHAPE);
+#define CALL(DT) hipLaunchKernelGGL((k_latent_store<DT>), dim3(b->n_tok), dim3(256), 0, (hipStream_t)s, proj, ld, (int)col0, weight, eps, (int)rank, \
+                                    (int)rot, freq, interleaved ? 1 : 0, (int)q_col0, (int)(rot ? heads : 0), (int)qdim, *b, cache);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
     return zl_launch_status();
+}
+
+extern "C" int zls_latent_store(const float* proj, int64_t ld, int64_t col0, const float* weight, float eps, int64_t rank, const zls_batch_t* b,
+                                void* cache, int dtype, zl_stream_t s) {
+    return zls_latent_rope_store(const_cast<float*>(proj), ld, col0, weight, eps, rank, 0, nullptr, 0, 0, 0, 0, b, cache, dtype, s);
 }
 
 extern "C" int64_t zls_latent_attention_workspace_bytes(int64_t n_tok, int64_t heads, int64_t rank, int64_t n_splits) {
@@ -587,7 +622,7 @@ extern "C" int64_t zls_latent_attention_workspace_bytes(int64_t n_tok, int64_t h
 extern "C" int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0, const float* gate, int64_t ldg, int64_t g_col0, const void* w_uk,
                                     const void* w_uv, const float* sink, const void* cache, const zls_batch_t* b, float scale, int64_t heads,
                                     int64_t dim, int64_t vdim, int64_t rank, void* out, int dtype, int single_only, void* workspace,
-                                    int64_t n_splits, int no_mfma, zl_stream_t s) {
+                                    int64_t n_splits, int no_mfma, int64_t window, zl_stream_t s) {
     ZL_CHECK_ARG(q && w_uk && w_uv && cache && out && workspace && seq_batch_ok(b) && b->page_table && b->page_size > 0 && b->max_pages > 0, ZL_EINVAL);
     ZL_CHECK_ARG(heads > 0 && dim > 0 && vdim > 0 && rank > 0 && heads <= 65535 && n_splits > 0 && n_splits <= 65535, ZL_EINVAL);
     ZL_CHECK_ARG(q_col0 >= 0 && q_col0 + heads * dim <= ldq && (!gate || (g_col0 >= 0 && g_col0 + heads <= ldg)), ZL_ESHAPE);
@@ -597,6 +632,8 @@ extern "C" int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0,
     p.q = q; p.gate = gate; p.w_uk = w_uk; p.w_uv = w_uv; p.sink = sink; p.cache = cache; p.out = out;
     p.ldq = ldq; p.ldg = ldg; p.q_col0 = (int)q_col0; p.g_col0 = (int)g_col0;
     p.heads = (int)heads; p.dim = (int)dim; p.vdim = (int)vdim; p.rank = (int)rank; p.scale = scale; p.single_only = single_only;
+    ZL_CHECK_ARG(window < (1 << 30), ZL_ESHAPE);
+    p.window = window > 0 ? (int)window : 0;
     p.vec = (rank % (dtype == ZL_BF16 ? 8 : 4) == 0 && ((uintptr_t)cache & 15) == 0) ? 1 : 0;
     const dim3 grid(b->n_tok, (unsigned)((heads + 3) / 4), (unsigned)n_splits);
     hipStream_t hs = (hipStream_t)s;
@@ -631,8 +668,8 @@ extern "C" int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0,
 extern "C" int zls_latent_attention_prompt(const float* q, int64_t ldq, int64_t q_col0, const float* gate, int64_t ldg, int64_t g_col0,
                                            const void* k, int64_t ldk, const void* vt, int64_t ldv, const float* sink, const int32_t* ctx_start,
                                            const zls_batch_t* b, float scale, int64_t heads, int64_t dim, int64_t vdim, void* out, int dtype,
-                                           zl_stream_t s) {
-    ZL_CHECK_ARG(q && k && vt && ctx_start && out && seq_batch_ok(b), ZL_EINVAL);
+                                           int64_t window, const int32_t* ctx_pos0, zl_stream_t s) {
+    ZL_CHECK_ARG(q && k && vt && ctx_start && out && seq_batch_ok(b) && window < (1 << 30), ZL_EINVAL);
     ZL_CHECK_ARG(dtype == ZL_BF16, ZL_EDTYPE);
     ZL_CHECK_ARG(heads > 0 && heads <= 65535 && dim > 0 && vdim > 0 && dim <= 256 && vdim <= 256, ZL_ESHAPE);
     ZL_CHECK_ARG(q_col0 >= 0 && q_col0 + heads * dim <= ldq && (!gate || (g_col0 >= 0 && g_col0 + heads <= ldg)), ZL_ESHAPE);
@@ -640,7 +677,7 @@ extern "C" int zls_latent_attention_prompt(const float* q, int64_t ldq, int64_t 
     FaP p;
     p.q = q; p.gate = gate; p.k = (const uint16_t*)k; p.vt = (const uint16_t*)vt; p.sink = sink; p.ctx_start = ctx_start; p.out = (uint16_t*)out;
     p.ldq = ldq; p.ldg = ldg; p.ldk = ldk; p.ldv = ldv; p.q_col0 = (int)q_col0; p.g_col0 = (int)g_col0;
-    p.heads = (int)heads; p.dim = (int)dim; p.vdim = (int)vdim; p.scale = scale;
+    p.heads = (int)heads; p.dim = (int)dim; p.vdim = (int)vdim; p.scale = scale; p.window = window > 0 ? (int)window : 0; p.ctx_pos0 = ctx_pos0;
     p.tiles_per_seq = (b->max_count + 63) / 64;
     p.vec_k = (dim % 8 == 0 && ldk % 8 == 0 && ((uintptr_t)k & 15) == 0) ? 1 : 0;
     const dim3 grid((unsigned)(b->n_seq * p.tiles_per_seq), (unsigned)heads);

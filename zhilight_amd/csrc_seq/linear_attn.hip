@@ -6,6 +6,8 @@
 //                       m is carried per sequence slot.
 // k_linear_attn_finish  a workgroup per (token, norm group): the optional division by max(|n . q|, exp(-m)) + den_eps per head, the RMS norm
 //                       over the group (all heads together, or each head alone), the weight, the sigmoid gate.
+// k_lowrank_decay      a decay per key channel from a low-rank projection: alpha = sigmoid(W2 u + bias)^(1 / tau), u the token's `low`
+//                       numbers; a workgroup per token, u in LDS, a thread per channel walks its row of W2 (fp32 sums)
 // Everything here is fp32; only the finished row is written in the serving format.
 #include "seq_common.h"
 
@@ -53,9 +55,25 @@ __global__ __launch_bounds__(kG) void k_exp_gates(const float* __restrict__ proj
     if (tid == 0) *ms = mm[0];
 }
 
+// alpha[t][c] = exp(log_sigmoid(sum_j w2[c][j] u[t][j] + bias[c]) / tau): the logarithm of the decay never leaves fp32
+template <int DT>
+__global__ __launch_bounds__(kG) void k_lowrank_decay(const float* __restrict__ proj, int64_t ld, int u_col0, int low, const void* __restrict__ w2,
+                                                      const float* __restrict__ bias, float inv_tau, int channels, float* __restrict__ alpha) {
+    extern __shared__ float us[];
+    const size_t t = blockIdx.x;
+    for (int j = threadIdx.x; j < low; j += kG) us[j] = proj[t * ld + u_col0 + j];
+    __syncthreads();
+    for (int c = threadIdx.x; c < channels; c += kG) {
+        float z = 0.f;
+        for (int j = 0; j < low; ++j) z = fmaf(SeqT<DT>::ld(w2, (size_t)c * low + j), us[j], z);
+        z += bias ? bias[c] : 0.f;
+        alpha[t * channels + c] = expf(log_sigmoid(z) * inv_tau);
+    }
+}
+
 struct FinP {
     const float* y; const float* m_vals; const float* weight; const float* gate; int64_t ldg;
-    int norm_col, heads, vdim, part, g_col0;
+    int norm_col, heads, vdim, part, g_col0, gate_kind;       // gate_kind 0: sigmoid(gate); 1: silu(gate)
     float q_scale, den_eps, eps;
     void* out;
 };
@@ -68,6 +86,7 @@ __global__ __launch_bounds__(kG) void k_linear_attn_finish(const FinP p) {
     auto value = [&](int c) {
         const int h = c / p.vdim, i = c % p.vdim;
         float v = yr[h * hp + i];
+        if (!p.m_vals) v *= p.q_scale;
         if (p.m_vals) {
             const float nq = yr[h * hp + p.vdim] * p.q_scale;
             v = v * p.q_scale / (fmaxf(fabsf(nq), expf(-p.m_vals[(size_t)t * p.heads + h])) + p.den_eps);
@@ -82,7 +101,10 @@ __global__ __launch_bounds__(kG) void k_linear_attn_finish(const FinP p) {
         const int c = c0 + i;
         float v = value(c) * f;
         if (p.weight) v *= p.weight[c];
-        if (p.gate) v *= seq_sigmoid(p.gate[(size_t)t * p.ldg + p.g_col0 + c]);
+        if (p.gate) {
+            const float gv = p.gate[(size_t)t * p.ldg + p.g_col0 + c];
+            v *= p.gate_kind == 1 ? seq_silu(gv) : seq_sigmoid(gv);
+        }
         SeqT<DT>::st(p.out, (size_t)t * p.heads * p.vdim + c, v);
     }
 }
@@ -100,14 +122,25 @@ extern "C" int zls_exp_gates(const float* proj, int64_t ld, int64_t i_col0, int6
 
 extern "C" int zls_linear_attn_finish(const float* y, int64_t norm_col, float q_scale, const float* m_vals, float den_eps, int64_t heads,
                                       int64_t vdim, int64_t norm_groups, const float* weight, float eps, const float* gate, int64_t ldg,
-                                      int64_t g_col0, int64_t n_tok, void* out, int dtype, zl_stream_t s) {
+                                      int64_t g_col0, int64_t n_tok, void* out, int dtype, int gate_kind, zl_stream_t s) {
     ZL_CHECK_ARG(y && out && heads > 0 && vdim > 0 && norm_groups > 0 && n_tok > 0 && (!m_vals || norm_col), ZL_EINVAL);
     ZL_CHECK_ARG((heads * vdim) % norm_groups == 0 && norm_groups <= 65535 && (!gate || (g_col0 >= 0 && g_col0 + heads * vdim <= ldg)), ZL_ESHAPE);
     FinP p;
     p.y = y; p.m_vals = m_vals; p.weight = weight; p.gate = gate; p.ldg = ldg; p.norm_col = norm_col ? 1 : 0; p.heads = (int)heads;
     p.vdim = (int)vdim; p.part = (int)(heads * vdim / norm_groups); p.g_col0 = (int)g_col0; p.q_scale = q_scale; p.den_eps = den_eps;
-    p.eps = eps; p.out = out;
+    p.eps = eps; p.out = out; p.gate_kind = gate_kind == 1 ? 1 : 0;
 #define CALL(DT) hipLaunchKernelGGL((k_linear_attn_finish<DT>), dim3((unsigned)n_tok, (unsigned)norm_groups), dim3(kG), 0, (hipStream_t)s, p);
+    ZLS_DISPATCH(dtype, CALL)
+#undef CALL
+    return zl_launch_status();
+}
+
+extern "C" int zls_lowrank_decay(const float* proj, int64_t ld, int64_t u_col0, int64_t low, const void* w2, const float* bias, float tau,
+                                 int64_t channels, int64_t n_tok, float* alpha, int dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(proj && w2 && alpha && low > 0 && channels > 0 && n_tok > 0 && tau > 0.f, ZL_EINVAL);
+    ZL_CHECK_ARG(u_col0 >= 0 && u_col0 + low <= ld && low <= 8192, ZL_ESHAPE);
+#define CALL(DT) hipLaunchKernelGGL((k_lowrank_decay<DT>), dim3((unsigned)n_tok), dim3(kG), (size_t)low * sizeof(float), (hipStream_t)s, proj, ld, \
+                                    (int)u_col0, (int)low, w2, bias, 1.0f / tau, (int)channels, alpha);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
     return zl_launch_status();

@@ -1,11 +1,13 @@
 // moe_seq.hip -- the routing side of a mixture-of-experts feed-forward over a ragged step (the products are zls_gemm_nt_grouped):
 //
-// k_moe_route    a wave per token: fp32 softmax over all router outputs, choice scores = probabilities + correction, group-limited choice
-//                (a group's score = its best choice score; outputs outside the best `keep` groups count as minus infinity), `top` picks by
-//                repeated arg-max (ties: the lower index), weights = the probabilities of the picks
+// k_moe_route    a wave per token: fp32 scores over all router outputs (softmax, or a sigmoid of each logit), choice scores = scores +
+//                correction, group-limited choice (a group's score = its best choice score, or the sum of its `group_top` best; outputs
+//                outside the best `keep` groups count as minus infinity), `top` picks by repeated arg-max (ties: the lower index),
+//                weights = the scores of the picks (optionally divided by their sum + renorm_eps)
 // k_moe_align    one workgroup: counts per expert, their prefix, every (token, choice) pair's place in the expert-sorted order, and the list of
 //                (expert, first, end) row tiles that the grouped product walks.  Identity outputs (id >= n_experts) take no place.
 // k_silu_mul     silu(gate) * up
+// k_act_mul      the gated activations of the feed-forwards: silu(g) u, gelu_tanh(g) u, or the clamped g sigmoid(a g) (u + 1)
 // k_moe_combine  a workgroup per token: the weighted sum of its picks' rows in the order of the picks; an identity pick adds the input row
 #include "seq_common.h"
 
@@ -21,7 +23,8 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {          // larg
 }
 
 __global__ __launch_bounds__(64) void k_moe_route(const float* __restrict__ logits, int n_out, const float* __restrict__ correction, int groups,
-                                                  int keep, int top, int renorm, int32_t* __restrict__ ids, float* __restrict__ weights) {
+                                                  int keep, int top, int renorm, int score_kind, int group_top, float renorm_eps,
+                                                  int32_t* __restrict__ ids, float* __restrict__ weights) {
     __shared__ float prob[1024], choice[1024], gscore[1024];
     const int t = blockIdx.x, lane = threadIdx.x;
     const float* z = logits + (size_t)t * n_out;
@@ -29,8 +32,13 @@ __global__ __launch_bounds__(64) void k_moe_route(const float* __restrict__ logi
     for (int i = lane; i < n_out; i += 64) mx = fmaxf(mx, z[i]);
     mx = zl_wave_max(mx);
     float sum = 0.f;
-    for (int i = lane; i < n_out; i += 64) { const float e = expf(z[i] - mx); prob[i] = e; sum += e; }
-    sum = zl_wave_sum(sum);
+    if (score_kind == 1) {                                               // every output on its own: sigmoid of its logit
+        for (int i = lane; i < n_out; i += 64) prob[i] = seq_sigmoid(z[i]);
+        sum = 1.0f;
+    } else {
+        for (int i = lane; i < n_out; i += 64) { const float e = expf(z[i] - mx); prob[i] = e; sum += e; }
+        sum = zl_wave_sum(sum);
+    }
     for (int i = lane; i < n_out; i += 64) {
         const float pr = prob[i] / sum;
         prob[i] = pr;
@@ -41,7 +49,21 @@ __global__ __launch_bounds__(64) void k_moe_route(const float* __restrict__ logi
         const int size = n_out / groups;
         for (int g = lane; g < groups; g += 64) {
             float best = -INFINITY;
-            for (int i = 0; i < size; ++i) best = fmaxf(best, choice[g * size + i]);
+            if (group_top <= 1) {
+                for (int i = 0; i < size; ++i) best = fmaxf(best, choice[g * size + i]);
+            } else {                                                     // the sum of the group's group_top largest choice scores
+                best = 0.f;
+                float bound = INFINITY; int bound_i = -1;                // the last one taken: the next is the largest below it (index order among equals)
+                for (int k = 0; k < group_top && k < size; ++k) {
+                    float bv = -INFINITY; int bi = -1;
+                    for (int i = 0; i < size; ++i) {
+                        const float v = choice[g * size + i];
+                        const bool below = v < bound || (v == bound && i > bound_i);
+                        if (below && (v > bv || bi < 0)) { bv = v; bi = i; }
+                    }
+                    best += bv; bound = bv; bound_i = bi;
+                }
+            }
             gscore[g] = best;
         }
         __syncthreads();
@@ -80,7 +102,7 @@ __global__ __launch_bounds__(64) void k_moe_route(const float* __restrict__ logi
     }
     if (renorm) {
         __syncthreads();
-        for (int k = lane; k < top; k += 64) weights[(size_t)t * top + k] /= wsum;
+        for (int k = lane; k < top; k += 64) weights[(size_t)t * top + k] /= wsum + renorm_eps;
     }
 }
 
@@ -150,6 +172,28 @@ __global__ __launch_bounds__(256) void k_silu_mul(const float* __restrict__ gu, 
     for (int c = threadIdx.x; c < ff; c += 256) SeqT<DT>::st(out, r * ff + c, seq_silu(gu[r * 2 * ff + c]) * gu[r * 2 * ff + ff + c]);
 }
 
+// kind 0: silu(g) u; 1: gelu_tanh(g) u; 2: g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit)
+__device__ __forceinline__ float gated_act(float g, float u, int kind, float alpha, float limit) {
+    if (kind == 1) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+    if (kind == 2) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        return g * seq_sigmoid(alpha * g) * (u + 1.0f);
+    }
+    return seq_silu(g) * u;
+}
+
+// block > 0: the row holds blocks of `block` gate columns followed by their `block` up columns; 0: all gates, then all ups
+template <int DT>
+__global__ __launch_bounds__(256) void k_act_mul(const float* __restrict__ gu, int ff, int kind, float alpha, float limit, int block,
+                                                 void* __restrict__ out) {
+    const size_t r = blockIdx.x;
+    for (int c = threadIdx.x; c < ff; c += 256) {
+        const int gi = block > 0 ? (c / block) * 2 * block + c % block : c, ui = block > 0 ? gi + block : ff + c;
+        SeqT<DT>::st(out, r * ff + c, gated_act(gu[r * 2 * ff + gi], gu[r * 2 * ff + ui], kind, alpha, limit));
+    }
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void k_moe_combine(const float* __restrict__ y, const int32_t* __restrict__ slot_pos, const int32_t* __restrict__ ids,
                                                      const float* __restrict__ weights, const void* __restrict__ h, int top, int n_experts, int width,
@@ -170,13 +214,14 @@ __global__ __launch_bounds__(256) void k_moe_combine(const float* __restrict__ y
 }  // namespace
 
 extern "C" int zls_moe_route(const float* logits, int64_t n_tok, int64_t n_out, const float* correction, int64_t groups, int64_t keep, int64_t top,
-                             int renorm, int32_t* ids, float* weights, zl_stream_t s) {
+                             int renorm, int score_kind, int64_t group_top, float renorm_eps, int32_t* ids, float* weights, zl_stream_t s) {
     ZL_CHECK_ARG(logits && ids && weights && n_tok > 0 && n_out > 0 && top > 0, ZL_EINVAL);
     ZL_CHECK_ARG(n_out <= 1024 && top <= n_out, ZL_ELIMIT);
     if (groups < 1) groups = 1;
     ZL_CHECK_ARG(n_out % groups == 0 && keep >= 1 && keep <= groups && top <= keep * (n_out / groups), ZL_ESHAPE);
+    ZL_CHECK_ARG((score_kind == 0 || score_kind == 1) && group_top >= 1, ZL_EINVAL);
     hipLaunchKernelGGL(k_moe_route, dim3((unsigned)n_tok), dim3(64), 0, (hipStream_t)s, logits, (int)n_out, correction, (int)groups, (int)keep,
-                       (int)top, renorm, ids, weights);
+                       (int)top, renorm, score_kind, (int)group_top, renorm_eps, ids, weights);
     return zl_launch_status();
 }
 
@@ -194,6 +239,15 @@ extern "C" int zls_moe_align(const int32_t* ids, int64_t n_slots, int64_t top, i
 extern "C" int zls_silu_mul(const float* gu, int64_t rows, int64_t ff, void* out, int dtype, zl_stream_t s) {
     ZL_CHECK_ARG(gu && out && rows > 0 && ff > 0, ZL_EINVAL);
 #define CALL(DT) hipLaunchKernelGGL((k_silu_mul<DT>), dim3((unsigned)rows), dim3(256), 0, (hipStream_t)s, gu, (int)ff, out);
+    ZLS_DISPATCH(dtype, CALL)
+#undef CALL
+    return zl_launch_status();
+}
+
+extern "C" int zls_act_mul(const float* gu, int64_t rows, int64_t ff, int kind, float alpha, float limit, int64_t block, void* out, int dtype,
+                           zl_stream_t s) {
+    ZL_CHECK_ARG(gu && out && rows > 0 && ff > 0 && kind >= 0 && kind <= 2 && block >= 0 && (block == 0 || ff % block == 0), ZL_EINVAL);
+#define CALL(DT) hipLaunchKernelGGL((k_act_mul<DT>), dim3((unsigned)rows), dim3(256), 0, (hipStream_t)s, gu, (int)ff, kind, alpha, limit, (int)block, out);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
     return zl_launch_status();

@@ -1,5 +1,6 @@
 // seq_elem.hip -- the per-token steps between the matrix products of a ragged step: embedding with learned positions, token shift with
-// its carried row, the scalar-gain RMS norm fused with the residual sum, the gathered final norm, PolyNorm.
+// its carried row, the scalar-gain RMS norm fused with the residual sum, the gathered final norm, PolyNorm, layer norm, the weighted RMS
+// norm before a sub-layer (alone, or fused with the residual sum that precedes it), scaled and soft-capped logits.
 // One workgroup per token row; every sum of squares is fp32 (butterfly inside a wave, waves in order).
 #include "seq_common.h"
 
@@ -127,6 +128,44 @@ __global__ __launch_bounds__(kT) void k_add_layer_norm(float* __restrict__ x, co
     for (int i = threadIdx.x; i < width; i += kT) SeqT<DT>::st(h2, row + i, (x[row + i] - mean) * inv * w2[i] + (bias2 ? bias2[i] : 0.f));
 }
 
+// x / sqrt(mean(x^2) + eps) * (w + shift): shift 1 for weights stored around zero, 0 for plain weights
+template <int DT>
+__global__ __launch_bounds__(kT) void k_rms_norm(const float* __restrict__ x, const int32_t* __restrict__ rows, const float* __restrict__ w,
+                                                 float shift, float eps, int width, void* __restrict__ out) {
+    __shared__ float red[16];
+    const float* r = x + (size_t)(rows ? rows[blockIdx.x] : (int)blockIdx.x) * width;
+    const size_t orow = (size_t)blockIdx.x * width;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += kT) ss = fmaf(r[i], r[i], ss);
+    const float f = 1.0f / sqrtf(zl_block_sum(ss, red) / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += kT) SeqT<DT>::st(out, orow + i, r[i] * f * (w[i] + shift));
+}
+
+// x += y (fp32, in place); optionally the NEXT sub-layer's input, the weighted RMS norm of the new row, in the serving format
+template <int DT>
+__global__ __launch_bounds__(kT) void k_add_rms_norm(float* __restrict__ x, const float* __restrict__ y, float eps, int width,
+                                                     const float* __restrict__ w2, float shift, void* __restrict__ h2) {
+    __shared__ float red[16];
+    const size_t row = (size_t)blockIdx.x * width;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += kT) {          // (a thread re-reads below only what it wrote itself)
+        const float v = x[row + i] + y[row + i];
+        x[row + i] = v;
+        ss = fmaf(v, v, ss);
+    }
+    if (!w2) return;
+    const float f = 1.0f / sqrtf(zl_block_sum(ss, red) / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += kT) SeqT<DT>::st(h2, row + i, x[row + i] * f * (w2[i] + shift));
+}
+
+// z <- cap * tanh(z * scale / cap) (cap <= 0: z * scale)
+__global__ __launch_bounds__(kT) void k_scale_softcap(float* __restrict__ z, int64_t n, float scale, float cap) {
+    const int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x;
+    if (i >= n) return;
+    const float v = z[i] * scale;
+    z[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
+}
+
 }  // namespace
 
 extern "C" int zls_embed(const int32_t* tokens, const void* table, const void* pos_table, int64_t vocab, int64_t max_positions, float scale,
@@ -190,5 +229,29 @@ extern "C" int zls_add_layer_norm(float* x, const float* y, const float* w, cons
 #define CALL(DT) hipLaunchKernelGGL((k_add_layer_norm<DT>), dim3((unsigned)rows), dim3(kT), 0, (hipStream_t)s, x, y, w, b, eps, (int)width, w2, b2, h2);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
+    return zl_launch_status();
+}
+
+extern "C" int zls_rms_norm(const float* x, const int32_t* rows, const float* w, float shift, float eps, int64_t n_rows, int64_t width, void* out,
+                            int dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(x && w && out && n_rows > 0 && width > 0, ZL_EINVAL);
+#define CALL(DT) hipLaunchKernelGGL((k_rms_norm<DT>), dim3((unsigned)n_rows), dim3(kT), 0, (hipStream_t)s, x, rows, w, shift, eps, (int)width, out);
+    ZLS_DISPATCH(dtype, CALL)
+#undef CALL
+    return zl_launch_status();
+}
+
+extern "C" int zls_add_rms_norm(float* x, const float* y, float eps, int64_t rows, int64_t width, const float* w2, float shift, void* h2, int dtype,
+                                zl_stream_t s) {
+    ZL_CHECK_ARG(x && y && rows > 0 && width > 0 && (!w2 || h2), ZL_EINVAL);
+#define CALL(DT) hipLaunchKernelGGL((k_add_rms_norm<DT>), dim3((unsigned)rows), dim3(kT), 0, (hipStream_t)s, x, y, eps, (int)width, w2, shift, h2);
+    ZLS_DISPATCH(dtype, CALL)
+#undef CALL
+    return zl_launch_status();
+}
+
+extern "C" int zls_scale_softcap(float* z, int64_t n, float scale, float cap, zl_stream_t s) {
+    ZL_CHECK_ARG(z && n > 0 && n < (1LL << 40), ZL_EINVAL);
+    hipLaunchKernelGGL(k_scale_softcap, dim3((unsigned)((n + kT - 1) / kT)), dim3(kT), 0, (hipStream_t)s, z, n, scale, cap);
     return zl_launch_status();
 }

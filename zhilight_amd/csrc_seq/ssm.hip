@@ -13,9 +13,12 @@
 
 namespace {
 
+// in_bias (nullable) is added to every INPUT of the convolution (the tail holds inputs with it; before a sequence's start the input is 0,
+// not the bias); act 0 leaves out the SiLU
 __global__ __launch_bounds__(256) void k_conv_silu(const float* __restrict__ proj, int64_t ld, int col0, const float* __restrict__ w,
-                                                   const float* __restrict__ bias, const float* __restrict__ tail, int channels, int taps,
-                                                   const zls_batch_t b, float* __restrict__ out) {
+                                                   const float* __restrict__ bias, const float* __restrict__ in_bias, int act,
+                                                   const float* __restrict__ tail, int channels, int taps, const zls_batch_t b,
+                                                   float* __restrict__ out) {
     const int t = blockIdx.x;
     const int sq = b.tok_seq[t];
     const int first = b.seq_start[sq];
@@ -23,26 +26,27 @@ __global__ __launch_bounds__(256) void k_conv_silu(const float* __restrict__ pro
     const float* tl = tail + (size_t)b.seq_slot[sq] * (taps - 1) * channels;
     for (int c = blockIdx.y * 256 + threadIdx.x; c < channels; c += gridDim.y * 256) {
         float a = bias ? bias[c] : 0.f;
+        const float ib = in_bias ? in_bias[c] : 0.f;
         for (int k = 0; k < taps; ++k) {
             const int back = taps - 1 - k;                             // the last column is the current token's
             const int src = i - back;
-            const float u = src >= 0 ? proj[(size_t)(first + src) * ld + col0 + c]
+            const float u = src >= 0 ? proj[(size_t)(first + src) * ld + col0 + c] + ib
                                      : tl[(size_t)(taps - 1 + src) * channels + c];     // src = -1 is the newest tail row
             a = fmaf(w[(size_t)c * taps + k], u, a);
         }
-        out[(size_t)t * channels + c] = seq_silu(a);
+        out[(size_t)t * channels + c] = act ? seq_silu(a) : a;
     }
 }
 
-__global__ __launch_bounds__(256) void k_conv_tail_update(const float* __restrict__ proj, int64_t ld, int col0, float* __restrict__ tail,
-                                                          int channels, int taps, const zls_batch_t b) {
+__global__ __launch_bounds__(256) void k_conv_tail_update(const float* __restrict__ proj, int64_t ld, int col0, const float* __restrict__ in_bias,
+                                                          float* __restrict__ tail, int channels, int taps, const zls_batch_t b) {
     const int sq = blockIdx.x;
     const int first = b.seq_start[sq], count = b.seq_start[sq + 1] - first;
     float* tl = tail + (size_t)b.seq_slot[sq] * (taps - 1) * channels;
     for (int c = blockIdx.y * 256 + threadIdx.x; c < channels; c += gridDim.y * 256) {
         for (int j = 0; j < taps - 1; ++j) {                           // new row j = input at portion index count - (taps - 1) + j
             const int src = count - (taps - 1) + j;
-            tl[(size_t)j * channels + c] = src >= 0 ? proj[(size_t)(first + src) * ld + col0 + c]
+            tl[(size_t)j * channels + c] = src >= 0 ? proj[(size_t)(first + src) * ld + col0 + c] + (in_bias ? in_bias[c] : 0.f)
                                                     : tl[(size_t)(taps - 1 + src) * channels + c];   // an older row j + count > j
         }
     }
@@ -62,6 +66,10 @@ struct ScanP {
     int kind, act, ones, q_col0, k_col0, v_col0;
     int cols;                                                // value columns per workgroup (all of them, or a part: blockIdx.z picks it)
     const float* decay_h; const float* decay_t; const float* gain_t;
+    // vec: the decay is a VECTOR per token, one number per state row (key channel): decay_v (n_tok, heads * n_state) fp32.  The staged row
+    // gets a third run [.. | a] laid out like B and C; a segment's decay product is then a vector too (k_seg_decay_prod), seg_prod
+    // (n_seq, n_seg, heads, n_state)
+    int vec; const float* decay_v;
 };
 
 constexpr int kScanSlots = 32;
@@ -74,10 +82,11 @@ constexpr int kScanSlots = 32;
 template <int NPT, int MAXT>
 __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batch_t b) {
     extern __shared__ float lds[];
-    const int P = p.vdim, N = p.n_state, W = P + 2 * N, KP = p.kp, CH = kScanSlots / KP;
+    const int NR = 2 + p.vec;                      // runs of n_state numbers behind x in a staged row
+    const int P = p.vdim, N = p.n_state, W = P + NR * N, KP = p.kp, CH = kScanSlots / KP;
     // a staged row in LDS: [x, padded to 4 | B: ngl groups of npt (+ 4 unused) | C: the same]: a thread's states are 16-byte aligned runs, the
     // runs of the ngl lanes of a column start 4 banks apart; everything no token writes (n >= N, the padding) is zero for good
-    const int P4 = (P + 3) & ~3, GS = p.npt + 4, WL = P4 + 2 * p.ngl * GS;
+    const int P4 = (P + 3) & ~3, GS = p.npt + 4, WL = P4 + NR * p.ngl * GS;
     float* rows = lds;                             // [CH][WL]
     float* dts = lds + CH * WL;                    // [CH] dt | [CH] decay
     for (int i = threadIdx.x; i < CH * WL; i += blockDim.x) rows[i] = 0.f;
@@ -106,11 +115,12 @@ __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batc
     }
     float prod = 1.0f;
     const float rate = lin ? 0.f : expf(p.a_log[h]), bias = lin ? 0.f : p.dt_bias[h], dskip = lin ? 0.f : p.d[h];
-    const float dec_h = (lin && !p.decay_t) ? p.decay_h[h] : 1.0f;
+    const float dec_h = (lin && !p.decay_t && p.decay_h) ? p.decay_h[h] : 1.0f;
     // slot u of a thread = (token u / KP of the chunk, column e = tid + (u % KP) * threads of the staged row): where it comes from inside
     // xbc and where it goes in LDS is the same for every chunk, so both offsets are worked out once (a wave64 VALU instruction costs four
     // cycles and this loop runs at one wave per SIMD: index arithmetic per chunk would cost more than the recurrence itself)
     int src_off[kScanSlots], dst_off[kScanSlots];
+    uint32_t from_dec = 0;                         // bit u: slot u is read from decay_v (rows of heads * N numbers)
 #pragma unroll
     for (int u = 0; u < kScanSlots; ++u) {
         const int i = u / KP, e = tid + (u % KP) * nthr;
@@ -119,6 +129,7 @@ __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batc
             const int n = (e - P) % N, half = (e - P) / N;
             col = lin ? (half ? p.q_col0 : p.k_col0) + h * N + n : inner + (half * p.groups + grp) * N + n;
             at = P4 + half * p.ngl * GS + (n / p.npt) * GS + n % p.npt;
+            if (half == 2 && e < W) { from_dec |= 1u << u; col = i * (p.heads * N - chan) + h * N + n; }     // (i * chan is added below)
         }
         src_off[u] = e < W ? ((lin && p.ones && e == P - 1) ? -2 : i * chan + col) : -1;      // -2: the column of ones
         dst_off[u] = i * WL + at;
@@ -127,8 +138,10 @@ __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batc
     auto fetch = [&](int c0) {
         const int cn = min(CH, count - c0);
         const float* base = srcbase + (size_t)(first + c0) * chan;
+        const float* dbase = p.vec ? p.decay_v + (size_t)(first + c0) * p.heads * N : base;
 #pragma unroll
-        for (int u = 0; u < kScanSlots; ++u) pre[u] = (u < cn * KP && src_off[u] >= 0) ? base[src_off[u]] : 1.0f;
+        for (int u = 0; u < kScanSlots; ++u)
+            pre[u] = (u < cn * KP && src_off[u] >= 0) ? ((from_dec >> u & 1u) ? dbase[src_off[u]] : base[src_off[u]]) : 1.0f;
         if (tid < cn) {
             if (lin) {
                 const size_t at = (size_t)(first + c0 + tid) * p.heads + h;
@@ -143,7 +156,7 @@ __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batc
         const int cn = min(CH, count - c0);
 #pragma unroll
         for (int u = 0; u < kScanSlots; ++u)
-            if (u < cn * KP && src_off[u] != -1) rows[dst_off[u]] = (p.act && src_off[u] >= 0) ? seq_silu(pre[u]) : pre[u];
+            if (u < cn * KP && src_off[u] != -1) rows[dst_off[u]] = (p.act && src_off[u] >= 0 && !(from_dec >> u & 1u)) ? seq_silu(pre[u]) : pre[u];
         if (tid < cn) {
             if (lin) {
                 dts[tid] = pre_dt;
@@ -171,15 +184,17 @@ __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batc
                 const float dx = dt * xv;
                 const float4* Bv = reinterpret_cast<const float4*>(row + P4 + g * GS);
                 const float4* Cv = reinterpret_cast<const float4*>(row + P4 + (p.ngl + g) * GS);
+                const float4* Av = reinterpret_cast<const float4*>(row + P4 + (2 * p.ngl + g) * GS);      // (read only with vec)
                 float part0 = 0.f, part1 = 0.f;
 #pragma unroll
                 for (int j = 0; j < NPT; j += 4) {
                     if (j < p.npt) {                               // (npt is a multiple of 4; states past N see B = C = 0 and stay 0)
                         const float4 bq = Bv[j >> 2], cq = Cv[j >> 2];
-                        S[j] = fmaf(decay, S[j], bq.x * dx);
-                        S[j + 1] = fmaf(decay, S[j + 1], bq.y * dx);
-                        S[j + 2] = fmaf(decay, S[j + 2], bq.z * dx);
-                        S[j + 3] = fmaf(decay, S[j + 3], bq.w * dx);
+                        const float4 aq = p.vec ? Av[j >> 2] : make_float4(decay, decay, decay, decay);
+                        S[j] = fmaf(aq.x, S[j], bq.x * dx);
+                        S[j + 1] = fmaf(aq.y, S[j + 1], bq.y * dx);
+                        S[j + 2] = fmaf(aq.z, S[j + 2], bq.z * dx);
+                        S[j + 3] = fmaf(aq.w, S[j + 3], bq.w * dx);
                         part0 = fmaf(S[j], cq.x, part0);
                         part1 = fmaf(S[j + 1], cq.y, part1);
                         part0 = fmaf(S[j + 2], cq.z, part0);
@@ -200,7 +215,22 @@ __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batc
         const int n = g * p.npt + j;
         if (j < p.npt && n < N) dst[(size_t)n * P + pp] = S[j];
     }
-    if (p.mode == 1 && tid == 0) p.seg_prod[seg_at] = prod;
+    if (p.mode == 1 && tid == 0 && !p.vec) p.seg_prod[seg_at] = prod;
+}
+
+// vector decays: the product of a segment's decays per (sequence, segment, head, state row), tokens in order; the last segment needs none
+__global__ __launch_bounds__(256) void k_seg_decay_prod(const ScanP p, const zls_batch_t b) {
+    const int sq = blockIdx.x / p.n_seg, seg = blockIdx.x % p.n_seg, h = blockIdx.y, N = p.n_state;
+    const int whole = b.seq_start[sq + 1] - b.seq_start[sq];
+    if ((seg + 1) * p.seg_len >= whole) return;
+    const int first = b.seq_start[sq] + seg * p.seg_len;
+    const size_t seg_at = ((size_t)sq * p.n_seg + seg) * p.heads + h;
+    for (int n = threadIdx.x; n < N; n += 256) {
+        float prod = 1.0f;
+        const float* a = p.decay_v + (size_t)first * p.heads * N + (size_t)h * N + n;
+        for (int i = 0; i < p.seg_len; ++i) prod *= a[(size_t)i * p.heads * N];
+        p.seg_prod[seg_at * N + n] = prod;
+    }
 }
 
 // start states of the segments 1 .. of every long portion: S_{k+1} = (product of segment k's decays) S_k + (segment k's end state from zero),
@@ -215,7 +245,7 @@ __global__ __launch_bounds__(256) void k_ssm_seg_combine(const ScanP p, const zl
         float S = st[e];
         for (int k = 0; k + 1 < nseg; ++k) {
             const size_t at = ((size_t)sq * p.n_seg + k) * p.heads + h;
-            S = fmaf(p.seg_prod[at], S, p.seg_state[at * NPs + e]);
+            S = fmaf(p.vec ? p.seg_prod[at * p.n_state + e / p.vdim] : p.seg_prod[at], S, p.seg_state[at * NPs + e]);
             p.seg_init[(at + p.heads) * NPs + e] = S;                   // segment k + 1 of the same sequence and head
         }
     }
@@ -239,30 +269,42 @@ __global__ __launch_bounds__(256) void k_gated_group_norm(const float* __restric
 
 }  // namespace
 
-extern "C" int zls_conv_silu(const float* proj, int64_t ld, int64_t col0, const float* w, const float* bias, const float* tail, int64_t channels,
-                             int64_t taps, const zls_batch_t* b, float* out, zl_stream_t s) {
+extern "C" int zls_short_conv(const float* proj, int64_t ld, int64_t col0, const float* w, const float* bias, const float* in_bias, int act,
+                              const float* tail, int64_t channels, int64_t taps, const zls_batch_t* b, float* out, zl_stream_t s) {
     ZL_CHECK_ARG(proj && w && out && seq_batch_ok(b) && channels > 0 && taps > 0 && (tail || taps == 1), ZL_EINVAL);
     ZL_CHECK_ARG(col0 >= 0 && col0 + channels <= ld, ZL_ESHAPE);
     const unsigned gy = (unsigned)((channels + 255) / 256 > 64 ? 64 : (channels + 255) / 256);
-    hipLaunchKernelGGL(k_conv_silu, dim3(b->n_tok, gy), dim3(256), 0, (hipStream_t)s, proj, ld, (int)col0, w, bias, tail, (int)channels, (int)taps, *b, out);
+    hipLaunchKernelGGL(k_conv_silu, dim3(b->n_tok, gy), dim3(256), 0, (hipStream_t)s, proj, ld, (int)col0, w, bias, in_bias, act ? 1 : 0, tail,
+                       (int)channels, (int)taps, *b, out);
     return zl_launch_status();
 }
 
-extern "C" int zls_conv_tail_update(const float* proj, int64_t ld, int64_t col0, float* tail, int64_t channels, int64_t taps, const zls_batch_t* b,
-                                    zl_stream_t s) {
+extern "C" int zls_conv_silu(const float* proj, int64_t ld, int64_t col0, const float* w, const float* bias, const float* tail, int64_t channels,
+                             int64_t taps, const zls_batch_t* b, float* out, zl_stream_t s) {
+    return zls_short_conv(proj, ld, col0, w, bias, nullptr, 1, tail, channels, taps, b, out, s);
+}
+
+extern "C" int zls_short_conv_tail(const float* proj, int64_t ld, int64_t col0, const float* in_bias, float* tail, int64_t channels, int64_t taps,
+                                   const zls_batch_t* b, zl_stream_t s) {
     ZL_CHECK_ARG(proj && seq_batch_ok(b) && channels > 0 && taps > 0, ZL_EINVAL);
     ZL_CHECK_ARG(col0 >= 0 && col0 + channels <= ld, ZL_ESHAPE);
     if (taps == 1) return ZL_OK;
     ZL_CHECK_ARG(tail, ZL_EINVAL);
     const unsigned gy = (unsigned)((channels + 255) / 256 > 64 ? 64 : (channels + 255) / 256);
-    hipLaunchKernelGGL(k_conv_tail_update, dim3(b->n_seq, gy), dim3(256), 0, (hipStream_t)s, proj, ld, (int)col0, tail, (int)channels, (int)taps, *b);
+    hipLaunchKernelGGL(k_conv_tail_update, dim3(b->n_seq, gy), dim3(256), 0, (hipStream_t)s, proj, ld, (int)col0, in_bias, tail, (int)channels,
+                       (int)taps, *b);
     return zl_launch_status();
+}
+
+extern "C" int zls_conv_tail_update(const float* proj, int64_t ld, int64_t col0, float* tail, int64_t channels, int64_t taps, const zls_batch_t* b,
+                                    zl_stream_t s) {
+    return zls_short_conv_tail(proj, ld, col0, nullptr, tail, channels, taps, b, s);
 }
 
 extern "C" int64_t zls_ssm_scan_workspace_bytes(int64_t n_seq, int64_t max_count, int64_t seg_len, int64_t heads, int64_t vdim, int64_t n_state) {
     if (n_seq <= 0 || max_count <= 0 || seg_len <= 0 || heads <= 0 || vdim <= 0 || n_state <= 0) return ZL_EINVAL;
     const int64_t n_seg = (max_count + seg_len - 1) / seg_len;
-    return n_seq * n_seg * heads * (2 * n_state * vdim + 1) * (int64_t)sizeof(float);
+    return n_seq * n_seg * heads * (2 * n_state * vdim + n_state + 1) * (int64_t)sizeof(float);      /* (room for a decay product per state row) */
 }
 
 // sizes the thread layout for (heads, vdim, n_state) in p and launches the scan (whole portions, or long ones in segments)
@@ -279,9 +321,10 @@ static int launch_scan(ScanP& p, int64_t heads, int64_t vdim, int64_t n_state, c
     const int64_t threads = (ngl * cols + 63) / 64 * 64;
     p.heads = (int)heads; p.vdim = (int)vdim; p.n_state = (int)n_state;
     p.ngl = (int)ngl; p.npt = (int)npt;
-    const int64_t row = vdim + 2 * n_state;
+    const int64_t runs = 2 + (p.vec ? 1 : 0);
+    const int64_t row = vdim + runs * n_state;
     int64_t kp = (row + threads - 1) / threads;                        // register slots a staged token row takes per thread
-    const size_t row_bytes = (size_t)((vdim + 3) / 4 * 4 + 2 * ngl * (npt + 4) + 2) * sizeof(float);
+    const size_t row_bytes = (size_t)((vdim + 3) / 4 * 4 + runs * ngl * (npt + 4) + 2) * sizeof(float);
     while (kp < kScanSlots && (kScanSlots / kp) * row_bytes > 64 * 1024) ++kp;      // long rows: fewer tokens staged at a time
     ZL_CHECK_ARG(kp <= kScanSlots, ZL_ELIMIT);
     p.kp = (int)kp;
@@ -315,6 +358,7 @@ static int launch_scan(ScanP& p, int64_t heads, int64_t vdim, int64_t n_state, c
     } else {
         p.mode = 1;
         SCAN_ANY
+        if (p.vec) hipLaunchKernelGGL(k_seg_decay_prod, dim3((unsigned)(b->n_seq * n_seg), (unsigned)heads), dim3(256), 0, hs, p, *b);
         const int64_t want_z = (1024 + b->n_seq * heads - 1) / (b->n_seq * heads), have_z = (n_state * vdim + 255) / 256;
         hipLaunchKernelGGL(k_ssm_seg_combine, dim3(b->n_seq, (unsigned)heads, (unsigned)(want_z < have_z ? want_z : have_z)), dim3(256), 0, hs, p, *b);
         p.mode = 2;
@@ -339,14 +383,15 @@ extern "C" int zls_ssm_scan(const float* xbc, const float* proj, int64_t ld, int
 
 extern "C" int zls_decay_scan(const float* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, int act, const float* decay_h,
                               const float* decay_t, const float* gain_t, int norm_col, float* state, int64_t heads, int64_t dim, int64_t vdim,
-                              const zls_batch_t* b, float* y, void* workspace, int64_t seg_len, zl_stream_t s) {
-    ZL_CHECK_ARG(proj && (decay_h || decay_t) && state && y && seq_batch_ok(b) && heads > 0 && dim > 0 && vdim > 0, ZL_EINVAL);
+                              const zls_batch_t* b, float* y, void* workspace, int64_t seg_len, const float* decay_v, zl_stream_t s) {
+    ZL_CHECK_ARG(proj && (decay_h || decay_t || decay_v) && state && y && seq_batch_ok(b) && heads > 0 && dim > 0 && vdim > 0, ZL_EINVAL);
+    ZL_CHECK_ARG(!decay_v || (!decay_h && !decay_t && heads * dim * (int64_t)kScanSlots < (1LL << 31)), ZL_EINVAL);
     ZL_CHECK_ARG(q_col0 >= 0 && q_col0 + heads * dim <= ld && k_col0 >= 0 && k_col0 + heads * dim <= ld && v_col0 >= 0 &&
                  v_col0 + heads * vdim <= ld && ld * kScanSlots < (1LL << 31), ZL_ESHAPE);
     ScanP p = {};
     p.proj = proj; p.state = state; p.y = y; p.ld = ld; p.groups = (int)heads;
     p.kind = 1; p.act = act ? 1 : 0; p.ones = norm_col ? 1 : 0; p.q_col0 = (int)q_col0; p.k_col0 = (int)k_col0; p.v_col0 = (int)v_col0;
-    p.decay_h = decay_h; p.decay_t = decay_t; p.gain_t = gain_t;
+    p.decay_h = decay_h; p.decay_t = decay_t; p.gain_t = gain_t; p.vec = decay_v ? 1 : 0; p.decay_v = decay_v;
     return launch_scan(p, heads, vdim + p.ones, dim, b, workspace, seg_len, s);
 }
 

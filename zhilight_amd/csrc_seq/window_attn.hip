@@ -1,6 +1,7 @@
 // window_attn.hip -- softmax attention over a paged key / value cache for a ragged step: rotary positions on a part of every query and key
-// head, unit-RMS queries and keys, values turned by their own position and the sums turned back, a sliding window, weights mixed across
-// heads after the softmax, a sigmoid gate per output coordinate.
+// head (pairs half a part apart, or neighbouring coordinates), unit-RMS queries and keys, values turned by their own position and the sums
+// turned back, values blended with another layer's values of the same token, a sliding window that may keep the sequence's first keys, a
+// learned sink in the softmax denominator, weights mixed across heads after the softmax, a sigmoid gate per output coordinate.
 //
 // k_rope_norm_store    a workgroup per token, a wave per head in turn: the head's coordinates in registers, rotated, normed, written back
 //                      (queries, fp32, in place) or to the token's row of the paged planes (keys, values; serving format)
@@ -23,9 +24,9 @@ constexpr int kChunk = 128;         // the largest page k_window_attention walks
 constexpr int kMaxV = 8;            // output coordinates per thread: (all_kv ? kv_heads : 1) * vdim <= 256 * kMaxV
 
 // one head of `size` coordinates in the lanes' registers (coordinate i in lane i % 64, register i / 64): rotate the first n_rot (pairs
-// i, i + n_rot / 2) by pos * freq[i], optionally divide by the root mean square; the result stays in v[]
+// i, i + n_rot / 2; interleaved: pairs 2i, 2i + 1) by pos * freq[i], optionally divide by the root mean square; the result stays in v[]
 __device__ __forceinline__ void rope_head(float* v, const float* src, int size, int n_rot, const float* __restrict__ freq, float pos, bool norm,
-                                          float eps, int lane) {
+                                          float eps, int lane, bool interleaved = false) {
     const int half = n_rot >> 1;
     float ss = 0.f;
 #pragma unroll
@@ -35,10 +36,10 @@ __device__ __forceinline__ void rope_head(float* v, const float* src, int size, 
         if (i < size) {
             o = src[i];
             if (i < n_rot) {
-                const bool lo = i < half;
-                const float other = src[lo ? i + half : i - half];
+                const bool lo = interleaved ? (i & 1) == 0 : i < half;
+                const float other = src[interleaved ? (i ^ 1) : (lo ? i + half : i - half)];
                 float sn, cs;
-                seq_sincos(pos * freq[lo ? i : i - half], &sn, &cs);
+                seq_sincos(pos * freq[interleaved ? (i >> 1) : (lo ? i : i - half)], &sn, &cs);
                 o = lo ? o * cs - other * sn : o * cs + other * sn;
             }
             ss = fmaf(o, o, ss);
@@ -58,6 +59,8 @@ struct RopeP {
     const float* qk_freq; const float* v_freq;
     float eps;
     void* k_cache; void* v_cache;
+    int interleaved;
+    const float* vmix_src; int64_t vmix_ld; int vmix_col0; float vmix_lambda;     // values <- (1 - lambda) values + lambda vmix_src[t][col0 ..]
 };
 
 template <int DT>
@@ -74,19 +77,25 @@ __global__ __launch_bounds__(256) void k_rope_norm_store(const RopeP p, const zl
     for (int h = wave; h < p.heads + 2 * n_kv; h += 4) {                 // (a wave owns its heads: no two waves touch the same numbers)
         if (h < p.heads) {
             float* q = row + p.q_col0 + h * p.dim;
-            rope_head(v, q, p.dim, p.rot_dims, p.qk_freq, pos, p.qk_norm != 0, p.eps, lane);
+            rope_head(v, q, p.dim, p.rot_dims, p.qk_freq, pos, p.qk_norm != 0, p.eps, lane, p.interleaved != 0);
 #pragma unroll
             for (int r = 0; r < kMaxE; ++r)
                 if (lane + 64 * r < p.dim) q[lane + 64 * r] = v[r];
         } else if (h < p.heads + n_kv) {
             const int c = h - p.heads;
-            rope_head(v, row + p.k_col0 + c * p.dim, p.dim, p.rot_dims, p.qk_freq, pos, p.qk_norm != 0, p.eps, lane);
+            rope_head(v, row + p.k_col0 + c * p.dim, p.dim, p.rot_dims, p.qk_freq, pos, p.qk_norm != 0, p.eps, lane, p.interleaved != 0);
 #pragma unroll
             for (int r = 0; r < kMaxE; ++r)
                 if (lane + 64 * r < p.dim) SeqT<DT>::st(p.k_cache, (crow * p.kv_heads + c) * p.dim + lane + 64 * r, v[r]);
         } else {
             const int c = h - p.heads - n_kv;
             rope_head(v, row + p.v_col0 + c * p.vdim, p.vdim, p.v_freq ? p.vdim : 0, p.v_freq, pos, false, 0.f, lane);
+            if (p.vmix_src) {
+                const float* other = p.vmix_src + (size_t)t * p.vmix_ld + p.vmix_col0 + c * p.vdim;
+#pragma unroll
+                for (int r = 0; r < kMaxE; ++r)
+                    if (lane + 64 * r < p.vdim) v[r] = (1.0f - p.vmix_lambda) * v[r] + p.vmix_lambda * other[lane + 64 * r];
+            }
 #pragma unroll
             for (int r = 0; r < kMaxE; ++r)
                 if (lane + 64 * r < p.vdim)                             // values lie transposed inside a page: (kv head, coordinate, key)
@@ -119,13 +128,14 @@ template <> struct Ld8<ZL_F32> {
 struct AttnP {
     const float* q; int64_t ldq; int q_col0;
     const void* k_cache; const void* v_cache;
-    float scale; int window, heads, kv_heads, dim, vdim, all_kv;
+    float scale; int window, keep_first, heads, kv_heads, dim, vdim, all_kv;    // keep_first: keys 0 .. keep_first - 1 stay visible behind the window
     float* acc; float* ml;                 // (n_tok, heads, n_splits, nv) partial sums | (n_tok, heads, n_splits, 2) their maximum and weight sum
     int n_splits, pages_per_split, single_only;
     const int32_t* tiles;                  // the matrix-core kernel: (first flat token, rows, sequence) per query tile
 };
 
-// split s of a token walks the pages first + s * pages_per_split .. of its window (first = the page of the window's oldest key), a page at a
+// A token's pages: those that only hold kept first keys (before the page of the window's oldest key), then the window's.  Split s walks
+// pages_per_split of that list from s * pages_per_split, a page at a
 // time: scores of the page's keys (a wave per key), weights with the running maximum -- 0 for keys outside the window or after the
 // token -- then every thread adds the WHOLE page of its value coordinates (the plane holds values transposed, 8 keys per 16-byte load).
 // What a split leaves is unnormalised: sum_j e^(s_j - m) v_j with m and sum_j e^(s_j - m); k_head_mix_gate merges the splits.
@@ -141,23 +151,25 @@ __global__ __launch_bounds__(256) void k_window_attention(const AttnP p, const z
     const int ps = b.page_size;
     const int pos = b.seq_pos0[sq] + (t - b.seq_start[sq]);
     const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+    const int wp0 = lo / ps, nkp = min((p.keep_first + ps - 1) / ps, wp0);   // kept pages before the window's first page
     const int c = g / (p.heads / p.kv_heads);
     const int nv = p.all_kv ? p.kv_heads * p.vdim : p.vdim, voff = p.all_kv ? 0 : c * p.vdim;
     const int32_t* pages = b.page_table + (size_t)sq * b.max_pages;
-    const int pg0 = lo / ps + sp * p.pages_per_split, pg1 = min(pos / ps, pg0 + p.pages_per_split - 1);
+    const int li0 = sp * p.pages_per_split, li1 = min(nkp + pos / ps - wp0, li0 + p.pages_per_split - 1);
     for (int i = tid; i < p.dim; i += 256) qs[i] = p.q[(size_t)t * p.ldq + p.q_col0 + g * p.dim + i] * p.scale;
     float A[kMaxV];
 #pragma unroll
     for (int r = 0; r < kMaxV; ++r) A[r] = 0.f;
     float m = -INFINITY, l = 0.f;
     __syncthreads();
-    for (int pg = pg0; pg <= pg1; ++pg) {
+    for (int li = li0; li <= li1; ++li) {
+        const int pg = li < nkp ? li : wp0 + li - nkp;
         const size_t page = (size_t)pages[pg];
         const int j0 = pg * ps;
         for (int jj = wave; jj < ps; jj += 4) {
             const int j = j0 + jj;
             float part = -INFINITY;
-            if (j >= lo && j <= pos) {                                    // (wave-uniform)
+            if (j <= pos && (j >= lo || j < p.keep_first)) {              // (wave-uniform)
                 const size_t at = ((page * ps + jj) * p.kv_heads + c) * p.dim;
                 part = 0.f;
                 for (int i = lane; i < p.dim; i += 64) part = fmaf(qs[i], SeqT<DT>::ld(p.k_cache, at + i), part);
@@ -168,7 +180,7 @@ __global__ __launch_bounds__(256) void k_window_attention(const AttnP p, const z
         __syncthreads();
         float cm = -INFINITY;
         for (int jj = tid; jj < ps; jj += 256) cm = fmaxf(cm, sc[jj]);
-        const float m_new = fmaxf(m, zl_block_max(cm, red));              // finite: the page holds a key of the window
+        const float m_new = fmaxf(m, zl_block_max(cm, red));              // finite: the page holds a visible key
         float psum = 0.f;
         for (int jj = tid; jj < ps; jj += 256) { const float e = expf(sc[jj] - m_new); sc[jj] = e; psum += e; }      // e^(-inf) = 0
         const float corr = expf(m - m_new);                               // (first page: 0, on sums that are 0)
@@ -236,7 +248,7 @@ __device__ __forceinline__ void split8(const float* v, uint4& hi, uint4& lo) {
 template <int KS>                       // 32-coordinate steps of the head size: dim <= 32 KS
 __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, const zls_batch_t b) {
     __shared__ uint4 pfrag[2][4][2][2][64];                              // [buffer][query block][key half][hi, lo][lane]
-    __shared__ float corr_s[2][64], l_s[64];
+    __shared__ float corr_s[2][64], l_s[64], m_s[64];
     const int tile = blockIdx.x, g = blockIdx.y, part = blockIdx.z;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nrow = lane & 15, kq = lane >> 4;
     const int t0 = p.tiles[3 * tile], rows = p.tiles[3 * tile + 1], sq = p.tiles[3 * tile + 2];
@@ -286,8 +298,12 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
                 kf[kb][ks] = (32 * ks + 8 * kq < d) ? *reinterpret_cast<const uint4*>(kr + 32 * ks) : make_uint4(0, 0, 0, 0);
         }
     };
-    load_keys(lo_key / 64);
-    for (int pg = lo_key / 64; pg <= pg_last; ++pg, buf ^= 1) {
+    // the tile's pages: those that only hold kept first keys, then the pages from the oldest key any of its queries sees in its window
+    const int wp0 = lo_key / 64, nkp = min((p.keep_first + 63) / 64, wp0), li_last = nkp + pg_last - wp0;
+    auto page_of = [&](int li) { return li < nkp ? li : wp0 + li - nkp; };
+    load_keys(page_of(0));
+    for (int li = 0; li <= li_last; ++li, buf ^= 1) {
+        const int pg = page_of(li);
         const size_t page = (size_t)pages[pg];
         // ---- scores of the wave's 16 queries against the page's 64 keys
         f4v st[4];
@@ -300,7 +316,7 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
                 st[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8v, kf[kb][ks]), __builtin_bit_cast(b8v, ql[ks]), st[kb], 0, 0, 0);
             }
         }
-        if (pg < pg_last) load_keys(pg + 1);
+        if (li < li_last) load_keys(page_of(li + 1));
         // st[kb][r]: key pg * 64 + 16 kb + 4 kq + r, query nrow
         float cm = -INFINITY;
         bool vis[4][4];
@@ -309,7 +325,7 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int j = pg * 64 + 16 * kb + 4 * kq + r;
-                vis[kb][r] = qok && j <= pq && (p.window <= 0 || pq - j < p.window);
+                vis[kb][r] = qok && j <= pq && (p.window <= 0 || pq - j < p.window || j < p.keep_first);
                 if (vis[kb][r]) cm = fmaxf(cm, st[kb][r]);
             }
         cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
@@ -374,14 +390,15 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
             }
         }
     }
-    if (kq == 0) l_s[qi] = l_run;
+    if (kq == 0) { l_s[qi] = l_run; m_s[qi] = m_run; }
     __syncthreads();
-    // acc[i][qb][r]: value coordinate 16 (block) + 4 kq + r of query 16 qb + nrow; split 0 of the token's partial sums, already normalised
+    // acc[i][qb][r]: value coordinate 16 (block) + 4 kq + r of query 16 qb + nrow; split 0 of the token's partial sums, unnormalised as the
+    // plain kernel leaves them, with (maximum, weight sum): k_head_mix_gate normalises (and counts a sink)
 #pragma unroll
     for (int qb = 0; qb < 4; ++qb) {
         const int row = 16 * qb + nrow;
         if (row >= rows) continue;
-        const float inv = 1.0f / l_s[row];
+        const float inv = 1.0f;
         float* out = p.acc + (((size_t)(t0 + row) * p.heads + g) * p.n_splits) * nv;
 #pragma unroll
         for (int i = 0; i < kItems; ++i) {
@@ -394,8 +411,8 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
         for (int e = tid; e < rows * p.n_splits; e += 256) {
             const int row = e / p.n_splits, sp = e % p.n_splits;
             float* mlp = p.ml + 2 * ((((size_t)(t0 + row) * p.heads + g) * p.n_splits) + sp);
-            mlp[0] = sp == 0 ? 0.f : -INFINITY;
-            mlp[1] = sp == 0 ? 1.f : 0.f;
+            mlp[0] = sp == 0 ? m_s[row] : -INFINITY;
+            mlp[1] = sp == 0 ? l_s[row] : 0.f;
         }
 }
 
@@ -403,6 +420,7 @@ struct MixP {
     const float* acc; const float* ml; const float* talk; const float* v_freq; const float* gate; int64_t ldg; int g_col0;
     int heads, kv_heads, vdim, n_splits;
     void* out;
+    const float* sink;                                                    // (heads) nullable: exp(sink_h) joins head h's denominator
 };
 
 // a workgroup per (token, key / value head c): the splits of every source head merged into LDS (for c's values only), then for the heads of
@@ -425,12 +443,12 @@ __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_b
     if (S > 1)
         for (int k = threadIdx.x >> 6; k < n_src; k += 4) {               // a wave per source head, a lane per split: all loads at once
             const float2* mlp = reinterpret_cast<const float2*>(p.ml) + ((size_t)t * p.heads + src0 + k) * S;
-            float M = -INFINITY;
+            float M = p.sink ? p.sink[src0 + k] : -INFINITY;
             for (int s = lane; s < S; s += 64) M = fmaxf(M, mlp[s].x);
             M = zl_wave_max(M);
             float L = 0.f;
             for (int s = lane; s < S; s += 64) { const float2 v = mlp[s]; L += v.y > 0.f ? v.y * expf(v.x - M) : 0.f; }
-            L = zl_wave_sum(L);
+            L = zl_wave_sum(L) + (p.sink ? expf(p.sink[src0 + k] - M) : 0.f);
             for (int s = lane; s < S; s += 64) { const float2 v = mlp[s]; wsp[k * S + s] = v.y > 0.f ? expf(v.x - M) / L : 0.f; }
         }
     if (p.talk)
@@ -448,9 +466,17 @@ __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_b
             src[r] = a + (size_t)(src0 + kk[r]) * S * nv + col0 + e % vd;
             v[r] = 0.f;
         }
-        if (S == 1) {                                                     // one split: its own weight sum normalises it
+        if (S == 1) {                                                     // one split: its own weight sum (and the sink) normalises it
 #pragma unroll
-            for (int r = 0; r < 8; ++r) v[r] = (1.0f / p.ml[2 * ((size_t)t * p.heads + src0 + kk[r]) + 1]) * *src[r];
+            for (int r = 0; r < 8; ++r) {
+                const float* mlp = p.ml + 2 * ((size_t)t * p.heads + src0 + kk[r]);
+                float f = 1.0f / mlp[1];
+                if (p.sink) {
+                    const float sk = p.sink[src0 + kk[r]], M = fmaxf(mlp[0], sk), e = expf(mlp[0] - M);
+                    f = e / (mlp[1] * e + expf(sk - M));
+                }
+                v[r] = f * *src[r];
+            }
         } else {
             for (int s = 0; s < S; ++s) {
                 float x[8];
@@ -507,6 +533,7 @@ __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_b
 
 extern "C" int zls_rope_norm_store(float* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, int64_t heads, int64_t kv_heads,
                                    int64_t dim, int64_t vdim, const float* qk_freq, int64_t rot_dims, const float* v_freq, float eps, int qk_norm,
+                                   int interleaved, const float* vmix_src, int64_t vmix_ld, int64_t vmix_col0, float vmix_lambda,
                                    const zls_batch_t* b, void* k_cache, void* v_cache, int dtype, zl_stream_t s) {
     ZL_CHECK_ARG(proj && seq_batch_ok(b) && b->page_table && b->page_size > 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0, ZL_EINVAL);
     ZL_CHECK_ARG((k_cache == nullptr) == (v_cache == nullptr), ZL_EINVAL);
@@ -518,6 +545,8 @@ extern "C" int zls_rope_norm_store(float* proj, int64_t ld, int64_t q_col0, int6
     p.proj = proj; p.ld = ld; p.q_col0 = (int)q_col0; p.k_col0 = (int)k_col0; p.v_col0 = (int)v_col0; p.heads = (int)heads;
     p.kv_heads = (int)kv_heads; p.dim = (int)dim; p.vdim = (int)vdim; p.rot_dims = (int)rot_dims; p.qk_norm = qk_norm; p.qk_freq = qk_freq;
     p.v_freq = v_freq; p.eps = eps; p.k_cache = k_cache; p.v_cache = v_cache;
+    ZL_CHECK_ARG(!vmix_src || (vmix_col0 >= 0 && vmix_col0 + kv_heads * vdim <= vmix_ld), ZL_ESHAPE);
+    p.interleaved = interleaved ? 1 : 0; p.vmix_src = vmix_src; p.vmix_ld = vmix_ld; p.vmix_col0 = (int)vmix_col0; p.vmix_lambda = vmix_lambda;
 #define CALL(DT) hipLaunchKernelGGL((k_rope_norm_store<DT>), dim3(b->n_tok), dim3(256), 0, (hipStream_t)s, p, *b);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
@@ -525,17 +554,19 @@ extern "C" int zls_rope_norm_store(float* proj, int64_t ld, int64_t q_col0, int6
 }
 
 extern "C" int zls_window_attention(const float* q, int64_t ldq, int64_t q_col0, const void* k_cache, const void* v_cache, const zls_batch_t* b,
-                                    float scale, int64_t window, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim, int all_kv, float* acc,
-                                    float* ml, int64_t n_splits, int64_t pages_per_split, int single_only, int dtype, zl_stream_t s) {
+                                    float scale, int64_t window, int64_t keep_first, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
+                                    int all_kv, float* acc, float* ml, int64_t n_splits, int64_t pages_per_split, int single_only, int dtype,
+                                    zl_stream_t s) {
     ZL_CHECK_ARG(q && k_cache && v_cache && acc && ml && seq_batch_ok(b) && b->page_table && b->page_size > 0, ZL_EINVAL);
     ZL_CHECK_ARG(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0 && heads <= 65535, ZL_ESHAPE);
-    ZL_CHECK_ARG(q_col0 >= 0 && q_col0 + heads * dim <= ldq && window < (1 << 30) && n_splits >= 1 && n_splits <= 65535 && pages_per_split >= 1,
-                 ZL_ESHAPE);
+    ZL_CHECK_ARG(q_col0 >= 0 && q_col0 + heads * dim <= ldq && window < (1 << 30) && n_splits >= 1 && n_splits <= 65535 && pages_per_split >= 1 &&
+                 keep_first >= 0 && keep_first < (1 << 30), ZL_ESHAPE);
     ZL_CHECK_ARG((all_kv ? kv_heads : 1) * vdim <= 256 * kMaxV && dim <= 8192 && b->page_size <= kChunk && b->page_size % 8 == 0, ZL_ELIMIT);
     AttnP p = {};
     p.q = q; p.ldq = ldq; p.q_col0 = (int)q_col0; p.k_cache = k_cache; p.v_cache = v_cache; p.scale = scale; p.window = (int)window;
     p.heads = (int)heads; p.kv_heads = (int)kv_heads; p.dim = (int)dim; p.vdim = (int)vdim; p.all_kv = all_kv ? 1 : 0; p.acc = acc; p.ml = ml;
     p.n_splits = (int)n_splits; p.pages_per_split = (int)pages_per_split; p.single_only = single_only ? 1 : 0;
+    p.keep_first = p.window > 0 ? (int)keep_first : 0;
     const size_t lds = (size_t)dim * sizeof(float);
 #define CALL(DT) hipLaunchKernelGGL((k_window_attention<DT>), dim3(b->n_tok, (unsigned)heads, (unsigned)n_splits), dim3(256), lds, (hipStream_t)s, p, *b);
     ZLS_DISPATCH(dtype, CALL)
@@ -544,18 +575,19 @@ extern "C" int zls_window_attention(const float* q, int64_t ldq, int64_t q_col0,
 }
 
 extern "C" int zls_window_attention_prompt(const float* q, int64_t ldq, int64_t q_col0, const void* k_cache, const void* v_cache,
-                                           const zls_batch_t* b, const int32_t* tiles, int64_t n_tiles, float scale, int64_t window, int64_t heads,
-                                           int64_t kv_heads, int64_t dim, int64_t vdim, int all_kv, float* acc, float* ml, int64_t n_splits,
+                                           const zls_batch_t* b, const int32_t* tiles, int64_t n_tiles, float scale, int64_t window,
+                                           int64_t keep_first, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim, int all_kv, float* acc, float* ml, int64_t n_splits,
                                            int dtype, zl_stream_t s) {
     ZL_CHECK_ARG(q && k_cache && v_cache && acc && ml && tiles && n_tiles > 0 && seq_batch_ok(b) && b->page_table, ZL_EINVAL);
     ZL_CHECK_ARG(dtype == ZL_BF16, ZL_EDTYPE);
     ZL_CHECK_ARG(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && heads <= 65535 && n_splits >= 1 && q_col0 >= 0 && q_col0 + heads * dim <= ldq,
                  ZL_ESHAPE);
-    ZL_CHECK_ARG(b->page_size == 64 && dim > 0 && dim % 8 == 0 && dim <= 256 && vdim > 0 && vdim % 16 == 0 && window < (1 << 30), ZL_ESHAPE);
+    ZL_CHECK_ARG(b->page_size == 64 && dim > 0 && dim % 8 == 0 && dim <= 256 && vdim > 0 && vdim % 16 == 0 && window < (1 << 30) &&
+                 keep_first >= 0 && keep_first < (1 << 30), ZL_ESHAPE);
     AttnP p = {};
     p.q = q; p.ldq = ldq; p.q_col0 = (int)q_col0; p.k_cache = k_cache; p.v_cache = v_cache; p.scale = scale; p.window = (int)window;
     p.heads = (int)heads; p.kv_heads = (int)kv_heads; p.dim = (int)dim; p.vdim = (int)vdim; p.all_kv = all_kv ? 1 : 0; p.acc = acc; p.ml = ml;
-    p.n_splits = (int)n_splits; p.tiles = tiles;
+    p.n_splits = (int)n_splits; p.tiles = tiles; p.keep_first = p.window > 0 ? (int)keep_first : 0;
     const int64_t n_blocks = (all_kv ? kv_heads : 1) * vdim / 16, parts = (n_blocks + 4 * kItems - 1) / (4 * kItems);
     ZL_CHECK_ARG(parts <= 65535, ZL_ELIMIT);
     const dim3 grid((unsigned)n_tiles, (unsigned)heads, (unsigned)parts);
@@ -571,8 +603,8 @@ extern "C" int zls_window_attention_prompt(const float* q, int64_t ldq, int64_t 
 }
 
 extern "C" int zls_head_mix_gate(const float* acc, const float* ml, int64_t n_splits, const float* talk, const float* v_freq, const float* gate,
-                                 int64_t ldg, int64_t g_col0, const zls_batch_t* b, int64_t heads, int64_t kv_heads, int64_t vdim, void* out,
-                                 int dtype, zl_stream_t s) {
+                                 int64_t ldg, int64_t g_col0, const float* sink, const zls_batch_t* b, int64_t heads, int64_t kv_heads, int64_t vdim,
+                                 void* out, int dtype, zl_stream_t s) {
     ZL_CHECK_ARG(acc && ml && out && seq_batch_ok(b) && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && vdim > 0 && n_splits >= 1, ZL_EINVAL);
     ZL_CHECK_ARG((!v_freq || vdim % 2 == 0) && (!gate || (g_col0 >= 0 && g_col0 + heads * vdim <= ldg)), ZL_ESHAPE);
     const int64_t n_src = talk ? heads : heads / kv_heads;
@@ -580,7 +612,7 @@ extern "C" int zls_head_mix_gate(const float* acc, const float* ml, int64_t n_sp
     ZL_CHECK_ARG(lds <= 64 * 1024 && kv_heads <= 65535, ZL_ELIMIT);
     MixP p;
     p.acc = acc; p.ml = ml; p.n_splits = (int)n_splits; p.talk = talk; p.v_freq = v_freq; p.gate = gate; p.ldg = ldg; p.g_col0 = (int)g_col0;
-    p.heads = (int)heads; p.kv_heads = (int)kv_heads; p.vdim = (int)vdim; p.out = out;
+    p.heads = (int)heads; p.kv_heads = (int)kv_heads; p.vdim = (int)vdim; p.out = out; p.sink = sink;
 #define CALL(DT) hipLaunchKernelGGL((k_head_mix_gate<DT>), dim3(b->n_tok, (unsigned)kv_heads), dim3(256), lds, (hipStream_t)s, p, *b);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL

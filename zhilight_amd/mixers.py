@@ -33,66 +33,90 @@ def _rand(gen, shape, std, dtype, device):
 
 
 class LatentAttention:
-    """Causal attention whose keys and values are up-projections of a cached, RMS-normed low-rank latent (no positional rotation); optional
-    learned per-head sink in the softmax denominator and per-head sigmoid output gate.
-    Tensors under `prefix`: q (heads*dim, width), dkv (rank, width), dkv.norm (rank), uk (heads*dim, rank), uv (heads*vdim, rank),
-    sink (heads), g (heads, width), o (width, heads*vdim).  q | dkv | g are fused into one product."""
+    """Causal attention whose keys and values are up-projections of a cached, RMS-normed low-rank latent; optional learned per-head sink in
+    the softmax denominator, per-head sigmoid output gate, sliding window (`window` > 0: position p sees p - window < j <= p), and a
+    ROTATED part: with rot_dim > 0 every query head has rot_dim more coordinates behind its `dim` unrotated ones, the down-projection
+    rot_dim more rows behind the latent -- one key part shared by all heads -- and both are turned by the position (neighbouring pairs
+    (2i, 2i + 1), angle p * rot_base^(-2i / rot_dim)); score = (q_plain . k_plain + q_rot . k_rot) * scale.  The cached row is [latent |
+    rotated key part]; the up-projections are widened on the host (identity columns in uk, zeros in uv), so the kernels see one latent of
+    rank + rot_dim numbers and heads of dim + rot_dim.
+    Tensors under `prefix`: q (heads*(dim+rot_dim), width), dkv (rank+rot_dim, width), dkv.norm (rank), uk (heads*dim, rank), uv (heads*vdim,
+    rank), sink (heads), g (heads, width), o (width, heads*vdim).  q | dkv | g are fused into one product."""
 
-    def __init__(self, name, width, heads, dim, vdim, rank, scale, eps, sink=True, gate=True):
+    def __init__(self, name, width, heads, dim, vdim, rank, scale, eps, sink=True, gate=True, rot_dim=0, rot_base=10000.0, window=0):
+        if rot_dim % 2 or rot_dim < 0 or window < 0:
+            raise ZLError("latent attention: the rotated part is even, the window not negative")
         self.name, self.width, self.heads, self.dim, self.vdim, self.rank = name, width, heads, dim, vdim, rank
         self.scale, self.eps, self.has_sink, self.has_gate = float(scale), float(eps), sink, gate
+        self.rot, self.rot_base, self.window = int(rot_dim), float(rot_base), int(window)
+        self.qdim, self.row = dim + self.rot, rank + self.rot      # a query head's size; a cached row's size
         self.cache = None
         self.prompt_kernel = True         # bf16 portions on the matrix-core kernel (False: everything on the latent-space kernel)
         self.decode_mfma = True           # bf16 single tokens: the split pass on the matrix cores (False: the fp32 VALU kernel)
 
+    def _widen(self, uk, uv):
+        """the up-projections over the cached row [latent | rotated key part]: a head's keys are [W_uk,h c | k_rot] (identity columns pass
+        the shared part through, exactly: 1.0 times a number, summed with zeros), its values ignore the part (zero columns)"""
+        H, d, v, r, t = self.heads, self.dim, self.vdim, self.rank, self.rot
+        if t == 0:
+            return uk.contiguous(), uv.contiguous()
+        k2 = torch.zeros((H, d + t, r + t), dtype=uk.dtype, device=uk.device)
+        k2[:, :d, :r] = uk.reshape(H, d, r)
+        k2[:, d:, r:] = torch.eye(t, dtype=uk.dtype, device=uk.device)
+        v2 = torch.zeros((H * v, r + t), dtype=uv.dtype, device=uv.device)
+        v2[:, :r] = uv
+        return k2.reshape(H * (d + t), r + t).contiguous(), v2.contiguous()
+
     def load(self, get, prefix, dtype, device):
         H, d, v, r, W = self.heads, self.dim, self.vdim, self.rank, self.width
-        parts = [_mat(get, prefix + "q", (H * d, W), dtype, device), _mat(get, prefix + "dkv", (r, W), dtype, device)]
+        parts = [_mat(get, prefix + "q", (H * self.qdim, W), dtype, device), _mat(get, prefix + "dkv", (self.row, W), dtype, device)]
         if self.has_gate:
             parts.append(_mat(get, prefix + "g", (H, W), dtype, device))
         self.w_in = torch.cat(parts, dim=0).contiguous()
         self.dkv_norm = _vec(get, prefix + "dkv.norm", r, device)
-        self.w_uk = _mat(get, prefix + "uk", (H * d, r), dtype, device)
-        self.w_uv = _mat(get, prefix + "uv", (H * v, r), dtype, device)
+        self.w_uk, self.w_uv = self._widen(_mat(get, prefix + "uk", (H * d, r), dtype, device), _mat(get, prefix + "uv", (H * v, r), dtype, device))
         self.sink = _vec(get, prefix + "sink", H, device) if self.has_sink else None
         self.w_o = _mat(get, prefix + "o", (W, H * v), dtype, device)
+        self.freq = rotary_frequencies(self.rot, self.rot_base, 1.0, device) if self.rot else None
         return self
 
     def init_random(self, gen, dtype, device):
         H, d, v, r, W = self.heads, self.dim, self.vdim, self.rank, self.width
-        self.w_in = _rand(gen, (H * d + r + (H if self.has_gate else 0), W), W ** -0.5, dtype, device)
+        self.w_in = _rand(gen, (H * self.qdim + self.row + (H if self.has_gate else 0), W), W ** -0.5, dtype, device)
         self.dkv_norm = torch.ones(r, device=device)
-        self.w_uk = _rand(gen, (H * d, r), r ** -0.5, dtype, device)
-        self.w_uv = _rand(gen, (H * v, r), r ** -0.5, dtype, device)
+        self.w_uk, self.w_uv = self._widen(_rand(gen, (H * d, r), r ** -0.5, dtype, device), _rand(gen, (H * v, r), r ** -0.5, dtype, device))
         self.sink = torch.zeros(H, device=device) if self.has_sink else None
         self.w_o = _rand(gen, (W, H * v), (H * v) ** -0.5, dtype, device)
+        self.freq = rotary_frequencies(self.rot, self.rot_base, 1.0, device) if self.rot else None
         return self
 
     def bind(self, cache, dtype):
-        self.cache = cache.add_plane(self.name + ".latent", (self.rank,), dtype)
+        self.cache = cache.add_plane(self.name + ".latent", (self.row,), dtype)
 
     def weight_bytes(self):
         return sum(t.numel() * t.element_size() for t in (self.w_in, self.w_uk, self.w_uv, self.w_o))
 
     def forward(self, h, batch):
-        H, d, r = self.heads, self.dim, self.rank
-        proj = seqops.gemm_nt(h, self.w_in)                                       # fp32 [q | latent | gate]
-        seqops.latent_store(proj, H * d, self.dkv_norm, self.eps, r, batch, self.cache)
+        H, d, r = self.heads, self.qdim, self.row                                # (sizes as the kernels see them: with the rotated part)
+        proj = seqops.gemm_nt(h, self.w_in)                                       # fp32 [q | latent, rotated key part | gate]
+        seqops.latent_store(proj, H * d, self.dkv_norm, self.eps, self.rank, batch, self.cache, rot=self.rot, freq=self.freq, interleaved=True,
+                            q_col0=0, heads=H, qdim=d)
         gate = proj if self.has_gate else None
         prompt = batch.n_ctx > 0 and self.prompt_kernel and h.dtype == torch.bfloat16 and max(d, self.vdim) <= 256
         a = torch.empty((batch.n_tok, H * self.vdim), dtype=h.dtype, device=h.device)
         if prompt:
-            # portions: keys and values of their contexts up-projected once (K = C W_uk^T, V^T = W_uv C^T, gathered from the pages), then
-            # the matrix-core kernel; single tokens stay on the latent-space kernel below
+            # portions: keys and values of their contexts (as far back as the window reaches) up-projected once (K = C W_uk^T, V^T = W_uv C^T,
+            # gathered from the pages), then the matrix-core kernel; single tokens stay on the latent-space kernel below
+            _, _, ctx_rows, n_ctx = batch.context(self.window)
             flat = self.cache.view(-1, r)
-            k = torch.empty((batch.n_ctx, H * d), dtype=h.dtype, device=h.device)
-            vt = torch.empty((H * self.vdim, batch.n_ctx), dtype=h.dtype, device=h.device)
-            seqops.gemm_nt_gather(flat, batch.ctx_rows, self.w_uk, None, batch.n_ctx, H * d, k)
-            seqops.gemm_nt_gather(self.w_uv, None, flat, batch.ctx_rows, H * self.vdim, batch.n_ctx, vt)
-            seqops.latent_attention_prompt(proj, 0, gate, H * d + r, k, vt, self.sink, batch, self.scale, H, d, self.vdim, a)
+            k = torch.empty((n_ctx, H * d), dtype=h.dtype, device=h.device)
+            vt = torch.empty((H * self.vdim, n_ctx), dtype=h.dtype, device=h.device)
+            seqops.gemm_nt_gather(flat, ctx_rows, self.w_uk, None, n_ctx, H * d, k)
+            seqops.gemm_nt_gather(self.w_uv, None, flat, ctx_rows, H * self.vdim, n_ctx, vt)
+            seqops.latent_attention_prompt(proj, 0, gate, H * d + r, k, vt, self.sink, batch, self.scale, H, d, self.vdim, a, window=self.window)
         if not prompt or batch.n_single:
             seqops.latent_attention(proj, 0, gate, H * d + r, self.w_uk, self.w_uv, self.sink, self.cache, batch, self.scale, H, d, self.vdim,
-                                    out=a, single_only=prompt, mfma=self.decode_mfma)
+                                    out=a, single_only=prompt, mfma=self.decode_mfma, window=self.window)
         return seqops.gemm_nt(a, self.w_o)
 
 
@@ -192,16 +216,32 @@ class WindowAttention:
         position (rotate_values; frequencies from the same base, never scaled),
       * the heads' softmax weights mixed by a (heads, heads) matrix after the softmax (tensor `talk`),
       * a sigmoid gate per output coordinate computed from the mixer's input (tensor `g`),
-      * keys and values borrowed from another layer's cache (kv_source: that layer's WindowAttention; then no k / v tensors).
+      * keys and values borrowed from another layer's cache (kv_source: that layer's WindowAttention; then no k / v tensors),
+      * rotated pairs that are neighbours (2i, 2i + 1) instead of (i, i + rot_dims / 2) (rope_interleaved),
+      * biases on q, k, v (bias; tensors q.b, k.b, v.b) and a short causal convolution over time on every channel of q, k, v right after the
+        projection (conv_taps > 0; tensors q.conv, k.conv, v.conv (channels, taps); the last taps - 1 projected rows are slot state),
+      * the sequence's first keep_first keys visible behind the window, at their true positions,
+      * a learned sink per head in the softmax denominator (tensor `sink`; no key, no value, not scaled),
+      * values blended with ANOTHER such layer's values of the same token before they are cached, v <- (1 - lam) v + lam v_other with lam
+        the scalar tensor `vmix` (v_mix_source: that layer's WindowAttention, which ran earlier in the same step).
     Tensors under `prefix`: q (heads*dim, width), k (kv_heads*dim, width), v (kv_heads*vdim, width), talk (heads, heads), g (heads*vdim, width),
     o (width, heads*vdim).  q | k | v | g are one product."""
 
     def __init__(self, name, width, heads, kv_heads, dim, vdim, scale, window, rot_dims, rot_base, rot_scaling, eps, qk_norm=True,
-                 rotate_values=True, talk=True, gate=True, kv_source=None):
+                 rotate_values=True, talk=True, gate=True, kv_source=None, rope_interleaved=False, bias=False, conv_taps=0, keep_first=0,
+                 sink=False, v_mix=False, v_mix_source=None):
         if heads % kv_heads or rot_dims % 2 or rot_dims > dim or (rotate_values and vdim % 2):
             raise ZLError("attention: heads must divide by kv_heads, rotated sizes must be even and fit the head")
         if kv_source is not None and (kv_source.kv_heads, kv_source.dim, kv_source.vdim) != (kv_heads, dim, vdim):
             raise ZLError("attention: a borrowed cache must have this layer's key / value shape")
+        if kv_source is not None and (bias or conv_taps or v_mix):
+            raise ZLError("attention: a layer that borrows keys and values has no key / value projections to bias, convolve or blend")
+        if v_mix_source is not None and (v_mix_source.kv_heads * v_mix_source.vdim != kv_heads * vdim):
+            raise ZLError("attention: blended values must have this layer's value shape")
+        self.interleaved, self.has_bias, self.taps, self.keep_first = bool(rope_interleaved), bool(bias), int(conv_taps), int(keep_first)
+        self.has_sink, self.v_mix, self.v_mix_source = bool(sink), bool(v_mix), v_mix_source
+        self.sink = self.in_bias = self.conv_w = self.tail = self.last_values = None
+        self.vmix_lambda = 0.0
         self.name, self.width, self.heads, self.kv_heads, self.dim, self.vdim = name, width, heads, kv_heads, dim, vdim
         self.scale, self.window, self.rot_dims, self.rot_base, self.rot_scaling = float(scale), int(window), rot_dims, float(rot_base), float(rot_scaling)
         self.eps, self.qk_norm, self.rotate_values, self.has_talk, self.has_gate = float(eps), qk_norm, rotate_values, talk, gate
@@ -231,6 +271,17 @@ class WindowAttention:
         self.w_in = torch.cat(parts, dim=0).contiguous()
         self.talk = _mat(get, prefix + "talk", (H, H), torch.float32, device) if self.has_talk else None
         self.w_o = _mat(get, prefix + "o", (W, H * v), dtype, device)
+        names = ("q", "k", "v") if self.kv_source is None else ("q",)
+        sizes = {"q": H * d, "k": G * d, "v": G * v}
+        if self.has_bias:
+            self.in_bias = torch.cat([_vec(get, prefix + n + ".b", sizes[n], device) for n in names]).contiguous()
+        if self.taps:
+            self.conv_w = torch.cat([_mat(get, prefix + n + ".conv", (sizes[n], self.taps), torch.float32, device) for n in names]).contiguous()
+        elif self.has_bias:
+            self.conv_w = torch.ones((sum(sizes[n] for n in names), 1), device=device)       # (one tap of weight 1: the bias alone)
+        self.sink = _vec(get, prefix + "sink", H, device) if self.has_sink else None
+        if self.v_mix:
+            self.vmix_lambda = float(_vec(get, prefix + "vmix", 1, device)[0])
         self._tables(device)
         return self
 
@@ -239,6 +290,15 @@ class WindowAttention:
         self.w_in = _rand(gen, (self._cols()[3], W), W ** -0.5, dtype, device)
         self.talk = (torch.eye(H, device=device) + 0.1 * torch.randn(H, H, generator=gen, device=device)) if self.has_talk else None
         self.w_o = _rand(gen, (W, H * v), (H * v) ** -0.5, dtype, device)
+        C = self._cols()[2]
+        if self.has_bias:
+            self.in_bias = 0.1 * torch.randn(C, generator=gen, device=device)
+        if self.taps:
+            self.conv_w = torch.randn(C, self.taps, generator=gen, device=device) * self.taps ** -0.5
+        elif self.has_bias:
+            self.conv_w = torch.ones((C, 1), device=device)
+        self.sink = torch.zeros(H, device=device) if self.has_sink else None
+        self.vmix_lambda = 0.5 if self.v_mix else 0.0
         self._tables(device)
         return self
 
@@ -248,6 +308,8 @@ class WindowAttention:
             return
         self.k_cache = cache.add_plane(self.name + ".k", (self.kv_heads * self.dim,), dtype)
         self.v_cache = cache.add_plane(self.name + ".v", (self.kv_heads * self.vdim,), dtype)      # (the kernels keep a page transposed)
+        if self.taps > 1:
+            self.tail = cache.add_state(self.name + ".conv", (self.taps - 1, self._cols()[2]))
 
     def weight_bytes(self):
         return sum(t.numel() * t.element_size() for t in (self.w_in, self.w_o))
@@ -257,11 +319,20 @@ class WindowAttention:
         k0, v0, g0, _ = self._cols()
         own = self.kv_source is None
         proj = seqops.gemm_nt(h, self.w_in)                                       # fp32 [q | k | v | gate]
-        seqops.rope_norm_store(proj, 0, k0, v0, H, G, d, v, self.qk_freq, self.rot_dims, self.v_freq, self.eps, self.qk_norm, batch,
-                               self.k_cache if own else None, self.v_cache if own else None)
-        acc, ml, n_splits = seqops.window_attention(proj, 0, self.k_cache, self.v_cache, batch, self.scale, self.window, H, G, d, v,
-                                                    all_kv=self.has_talk, mfma=self.prompt_kernel, n_splits=self.n_splits)
-        a = seqops.head_mix_gate(acc, ml, n_splits, self.talk, self.v_freq, proj if self.has_gate else None, g0, batch, H, G, v, h.dtype)
+        # biases and the short convolution give a second buffer [q | k | v] (the gate stays in proj); otherwise q is rotated inside proj
+        qkv = seqops.short_conv(proj, 0, self.conv_w, self.in_bias, self.tail, batch) if self.conv_w is not None else proj
+        blend = None
+        if self.v_mix and self.v_mix_source is not None:
+            src, col = self.v_mix_source.last_values
+            blend = (src, col, self.vmix_lambda)
+        self.last_values = (qkv, v0) if self.v_mix else None                      # (this step's values before blending, for a later layer)
+        seqops.rope_norm_store(qkv, 0, k0, v0, H, G, d, v, self.qk_freq, self.rot_dims, self.v_freq, self.eps, self.qk_norm, batch,
+                               self.k_cache if own else None, self.v_cache if own else None, interleaved=self.interleaved, vmix=blend)
+        acc, ml, n_splits = seqops.window_attention(qkv, 0, self.k_cache, self.v_cache, batch, self.scale, self.window, H, G, d, v,
+                                                    all_kv=self.has_talk, mfma=self.prompt_kernel, n_splits=self.n_splits,
+                                                    keep_first=self.keep_first)
+        a = seqops.head_mix_gate(acc, ml, n_splits, self.talk, self.v_freq, proj if self.has_gate else None, g0, batch, H, G, v, h.dtype,
+                                 sink=self.sink)
         return seqops.gemm_nt(a, self.w_o)
 
 
@@ -307,6 +378,89 @@ class DecayLinearAttention:
                               seg_len=self.scan_segment)
         a = seqops.linear_attn_finish(y, False, 1.0, None, 0.0, H, v, self.norm_groups, self.norm_w, self.eps, proj, 2 * H * d + H * v, h.dtype)
         return seqops.gemm_nt(a, self.w_o)
+
+
+class GatedLinearAttention:
+    """Linear attention with a learned decay per KEY CHANNEL and token: q = W_q h * dim^-1/2, k = W_k h, v = W_v h;
+        alpha = sigmoid(W_a2 (W_a1 h) + b)^(1 / tau)   (heads x dim, from a low-rank pair of projections)
+        S_t = diag(alpha_t) S_{t-1} + k_t v_t^T,  o_t = S_t^T q_t   per head, S fp32 per sequence, from zero
+    then each head's o divided by its root mean square over vdim, times a weight shared by the heads, times silu(W_g h), and the output
+    projection.  The logarithm of the decay, the decay and the recurrence are fp32; the scale dim^-1/2 is applied to o (the recurrence is
+    linear in q).  Tensors under `prefix`: q, k (heads*dim, width), v, g (heads*vdim, width), a1 (low, width), a2 (heads*dim, low), a2.b
+    (heads*dim), norm (vdim), o (width, heads*vdim).  q | k | v | g | a1 are one product."""
+
+    def __init__(self, name, width, heads, dim, vdim, tau, eps):
+        if tau <= 0:
+            raise ZLError("gated linear attention: tau > 0")
+        self.name, self.width, self.heads, self.dim, self.vdim = name, width, heads, dim, vdim
+        self.tau, self.eps = float(tau), float(eps)
+        self.scan_segment = None
+
+    def load(self, get, prefix, dtype, device):
+        H, d, v, W = self.heads, self.dim, self.vdim, self.width
+        a1 = get(prefix + "a1")
+        self.low = int(a1.shape[0])
+        self.w_in = torch.cat([_mat(get, prefix + "q", (H * d, W), dtype, device), _mat(get, prefix + "k", (H * d, W), dtype, device),
+                               _mat(get, prefix + "v", (H * v, W), dtype, device), _mat(get, prefix + "g", (H * v, W), dtype, device),
+                               _mat(get, prefix + "a1", (self.low, W), dtype, device)], dim=0).contiguous()
+        self.w_a2 = _mat(get, prefix + "a2", (H * d, self.low), dtype, device)
+        self.a2_bias = _vec(get, prefix + "a2.b", H * d, device)
+        self.norm_w = _vec(get, prefix + "norm", v, device).repeat(H).contiguous()
+        self.w_o = _mat(get, prefix + "o", (W, H * v), dtype, device)
+        return self
+
+    def init_random(self, gen, dtype, device, low=16):
+        H, d, v, W = self.heads, self.dim, self.vdim, self.width
+        self.low = low
+        self.w_in = _rand(gen, (2 * H * d + 2 * H * v + low, W), W ** -0.5, dtype, device)
+        self.w_a2 = _rand(gen, (H * d, low), low ** -0.5, dtype, device)
+        self.a2_bias = torch.full((H * d,), 2.0, device=device)
+        self.norm_w = torch.ones(H * v, device=device)
+        self.w_o = _rand(gen, (W, H * v), (H * v) ** -0.5, dtype, device)
+        return self
+
+    def bind(self, cache, dtype):
+        self.state = cache.add_state(self.name + ".S", (self.heads, self.dim, self.vdim))
+
+    def weight_bytes(self):
+        return sum(t.numel() * t.element_size() for t in (self.w_in, self.w_a2, self.w_o))
+
+    def forward(self, h, batch):
+        H, d, v = self.heads, self.dim, self.vdim
+        proj = seqops.gemm_nt(h, self.w_in)                                       # fp32 [q | k | v | gate | low-rank decay input]
+        g0 = 2 * H * d + H * v
+        alpha = seqops.lowrank_decay(proj, g0 + H * v, self.w_a2, self.a2_bias, self.tau)
+        y = seqops.decay_scan(proj, 0, H * d, 2 * H * d, False, None, None, None, False, self.state, H, d, v, batch, seg_len=self.scan_segment,
+                              decay_v=alpha)
+        a = seqops.linear_attn_finish(y, False, d ** -0.5, None, 0.0, H, v, H, self.norm_w, self.eps, proj, g0, h.dtype, gate_act="silu")
+        return seqops.gemm_nt(a, self.w_o)
+
+
+class GatedFF:
+    """Dense gated feed-forward down(act(gate h) * (up h)) without biases; act: "gelu_tanh" (the tanh form) or "silu".
+    Tensors under `prefix`: gate, up (ff, width), down (width, ff).  gate | up are one product."""
+
+    def __init__(self, width, ff, act="gelu_tanh"):
+        if act not in ("gelu_tanh", "silu"):
+            raise ZLError(f"feed-forward: unknown activation {act!r}")
+        self.width, self.ff, self.act = width, ff, act
+
+    def load(self, get, prefix, dtype, device):
+        self.w_gu = torch.cat([_mat(get, prefix + "gate", (self.ff, self.width), dtype, device),
+                               _mat(get, prefix + "up", (self.ff, self.width), dtype, device)], dim=0).contiguous()
+        self.w_down = _mat(get, prefix + "down", (self.width, self.ff), dtype, device)
+        return self
+
+    def init_random(self, gen, dtype, device):
+        self.w_gu = _rand(gen, (2 * self.ff, self.width), self.width ** -0.5, dtype, device)
+        self.w_down = _rand(gen, (self.width, self.ff), self.ff ** -0.5, dtype, device)
+        return self
+
+    def weight_bytes(self):
+        return sum(t.numel() * t.element_size() for t in (self.w_gu, self.w_down))
+
+    def forward(self, h):
+        return seqops.gemm_nt(seqops.act_mul(seqops.gemm_nt(h, self.w_gu), h.dtype, kind=self.act), self.w_down)
 
 
 class MLSTMMixer:
@@ -369,18 +523,27 @@ class RoutedExpertsFF:
     e<j>.down (width, ff).  Gate and up rows of all experts are stacked in blocks of 16 (16 gate rows, their 16 up rows), so that the grouped
     product's epilogue finishes the activation."""
 
-    def __init__(self, width, ff, experts, top, identity=0, groups=1, keep=1, correction=True, renorm=False):
+    def __init__(self, width, ff, experts, top, identity=0, groups=1, keep=1, correction=True, renorm=False, score="softmax", group_top=1,
+                 renorm_eps=0.0, act="silu", act_alpha=1.0, limit=0.0):
+        """score: "softmax" over all outputs or "sigmoid" of each logit; group_top: a group scores by the sum of its group_top best choice
+        scores; act: "silu" -- silu(gate) up --, or "swish_clamp" -- g sigmoid(act_alpha g) (u + 1) with g = min(gate, limit),
+        u = clamp(up, -limit, limit)"""
+        if score not in ("softmax", "sigmoid") or act not in ("silu", "swish_clamp") or group_top < 1:
+            raise ZLError("experts: unknown score function or activation")
+        self.score, self.group_top, self.renorm_eps, self.act, self.act_alpha, self.limit = score, int(group_top), float(renorm_eps), act, \
+            float(act_alpha), float(limit)
         total = experts + identity
         if groups < 1 or total % groups or not 1 <= keep <= groups or top > keep * (total // groups):
             raise ZLError("experts: groups must divide the router outputs, and the kept groups must hold `top` outputs")
         self.width, self.ff, self.experts, self.top, self.identity = width, ff, experts, top, identity
         self.groups, self.keep, self.has_correction, self.renorm = groups, keep, correction, renorm
-        self.fused_act = ff % 16 == 0
+        self.packed = ff % 16 == 0                       # gate / up rows in blocks of 16: what the gated epilogue reads
+        self.fused_act = self.packed and act == "silu"   # (the products' epilogue knows silu(gate) * up; other activations take one more launch)
         self.few_rows = seqops.MOE_FEW_ROWS
         self.tile_m = None                # rows per expert tile of the grouped products (None: by the experts' average share)
 
     def _pack_gate_up(self, gate, up):
-        if not self.fused_act:
+        if not self.packed:
             return torch.cat([gate, up], dim=0)
         f, w = gate.shape
         return torch.stack([gate.reshape(f // 16, 16, w), up.reshape(f // 16, 16, w)], dim=1).reshape(2 * f, w)
@@ -410,13 +573,15 @@ class RoutedExpertsFF:
 
     def forward(self, h):
         logits = seqops.gemm_nt(h, self.w_router)                                 # fp32 sums of the products
-        ids, weights = seqops.moe_route(logits, self.correction, self.groups, self.keep, self.top, self.renorm)
+        ids, weights = seqops.moe_route(logits, self.correction, self.groups, self.keep, self.top, self.renorm, score=self.score,
+                                        group_top=self.group_top, renorm_eps=self.renorm_eps)
         sorted_tok, slot_pos, tiles, max_tiles, sorted_exp, tm = seqops.moe_align(ids, self.experts, self.tile_m)
         n_slots = ids.numel()
         few = sorted_exp if n_slots <= self.few_rows else None                    # decode steps: weight rows streamed per (row, column)
         if self.fused_act:
             a = seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots, gated=True, out_dtype=h.dtype, row_expert=few, tile_m=tm)
         else:
-            a = seqops.silu_mul(seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots, row_expert=few, tile_m=tm), h.dtype)
+            a = seqops.act_mul(seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots, row_expert=few, tile_m=tm), h.dtype,
+                               kind=self.act, alpha=self.act_alpha, limit=self.limit, block=16 if self.packed else 0)
         y = seqops.gemm_nt_grouped(a, None, self.w_down, tiles, max_tiles, n_slots, row_expert=few, tile_m=tm)
         return seqops.moe_combine(y, slot_pos, ids, weights, h, self.experts)

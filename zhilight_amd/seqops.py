@@ -19,7 +19,8 @@ SYMBOLS = ["zls_version", "zls_gemm_nt", "zls_embed", "zls_token_shift", "zls_ad
            "zls_latent_store", "zls_latent_attention", "zls_latent_attention_workspace_bytes", "zls_latent_attention_prompt", "zls_gemm_nt_gather",
            "zls_conv_silu", "zls_conv_tail_update", "zls_ssm_scan", "zls_ssm_scan_workspace_bytes", "zls_gated_group_norm", "zls_layer_norm",
            "zls_add_layer_norm", "zls_rope_norm_store", "zls_window_attention", "zls_window_attention_prompt", "zls_head_mix_gate", "zls_decay_scan", "zls_exp_gates",
-           "zls_linear_attn_finish", "zls_moe_route", "zls_moe_align", "zls_gemm_nt_grouped", "zls_silu_mul", "zls_moe_combine"]
+           "zls_linear_attn_finish", "zls_moe_route", "zls_moe_align", "zls_gemm_nt_grouped", "zls_silu_mul", "zls_moe_combine", "zls_rms_norm",
+           "zls_add_rms_norm", "zls_scale_softcap", "zls_act_mul", "zls_short_conv", "zls_short_conv_tail", "zls_lowrank_decay", "zls_latent_rope_store"]
 _STATUS = {-1: "invalid argument (null pointer / non-positive size)", -2: "shape not supported", -3: "dtype not supported",
            -4: "exceeds a hardware limit"}
 
@@ -143,6 +144,31 @@ class RaggedBatch:
         self.max_ctx = max(s[0] + s[1] for s in seqs)
         self.c = Batch(n_seq, self.n_tok, max_pages, page_size, max(self.counts), 0, *[base + 4 * x for x in o])
         self.ref = C.byref(self.c)
+        self._seqs, self._windowed = seqs, {}
+
+    def context(self, window):
+        """(ctx_start, ctx_pos0, ctx_rows, n_ctx) for portions that look back `window` positions only: the cached rows from the 64-aligned
+        position at or below the oldest key the portion's first token sees, each sequence padded to a multiple of 64 rows.  window 0: the
+        whole context (ctx_pos0 None).  One more small host-to-device copy per distinct window of a step."""
+        if window <= 0:
+            return self.ctx_start, None, self.ctx_rows, self.n_ctx
+        if window not in self._windowed:
+            ps = self.c.page_size
+            ctx_rows, ctx_start, ctx_pos0 = [], [], []
+            for count, pos0, slot, pages in self._seqs:
+                if count == 1:
+                    ctx_start.append(-1)
+                    ctx_pos0.append(0)
+                    continue
+                c0 = max(0, pos0 - window + 1) // 64 * 64
+                ctx_start.append(len(ctx_rows))
+                ctx_pos0.append(c0)
+                rows = [pages[j // ps] * ps + j % ps for j in range(c0, pos0 + count)]
+                ctx_rows += rows + [rows[0]] * (-len(rows) % 64)
+            dev = torch.tensor(ctx_start + ctx_pos0 + ctx_rows, dtype=torch.int32).to(self.dev.device)
+            n = self.n_seq
+            self._windowed[window] = (dev[:n], dev[n:2 * n], dev[2 * n:], len(ctx_rows))
+        return self._windowed[window]
 
 
 def gemm_nt(x, w, out=None, out_dtype=torch.float32):
@@ -219,13 +245,18 @@ def polynorm(z, coef, eps, dtype):
     return out
 
 
-def latent_store(proj, col0, weight, eps, rank, batch, cache):
-    _cuda(proj, weight, cache)
-    _f32(proj, weight)
-    if cache.dim() != 3 or cache.shape[1] != batch.c.page_size or cache.shape[2] != rank or weight.numel() != rank:
-        raise ZLError("latent_store: cache must be (pages, page_size, rank)")
-    check(lib().zls_latent_store(_p(proj), _i(proj.shape[1]), _i(col0), _p(weight), _f(eps), _i(rank), batch.ref, _p(cache),
-                                 C.c_int(dt_code(cache.dtype)), _stream()), "latent_store")
+def latent_store(proj, col0, weight, eps, rank, batch, cache, rot=0, freq=None, interleaved=True, q_col0=0, heads=0, qdim=0):
+    """normed latent -> the tokens' cache rows; rot > 0: the `rot` columns behind the latent (one key part for all heads) are turned by the
+    position and stored behind it, and the last rot of the qdim coordinates of every query head (from q_col0) are turned in place"""
+    _cuda(proj, weight, cache, freq)
+    _f32(proj, weight, freq)
+    if cache.dim() != 3 or cache.shape[1] != batch.c.page_size or cache.shape[2] != rank + rot or weight.numel() != rank:
+        raise ZLError("latent_store: cache must be (pages, page_size, rank + rot)")
+    if rot and (freq is None or freq.numel() != rot // 2):
+        raise ZLError("latent_store: one frequency per rotated pair")
+    check(lib().zls_latent_rope_store(_p(proj), _i(proj.shape[1]), _i(col0), _p(weight), _f(eps), _i(rank), _i(rot), _p(freq),
+                                      C.c_int(int(interleaved)), _i(q_col0), _i(heads), _i(qdim), batch.ref, _p(cache),
+                                      C.c_int(dt_code(cache.dtype)), _stream()), "latent_store")
 
 
 def gemm_nt_gather(x, x_rows, w, w_rows, m, n, out):
@@ -241,19 +272,21 @@ def gemm_nt_gather(x, x_rows, w, w_rows, m, n, out):
     return out
 
 
-def latent_attention_prompt(q, q_col0, gate, g_col0, k, vt, sink, batch, scale, heads, dim, vdim, out):
-    """the portions of the step on the matrix cores; k (n_ctx, heads * dim), vt (heads * vdim, n_ctx) from gemm_nt_gather; writes its rows of out"""
+def latent_attention_prompt(q, q_col0, gate, g_col0, k, vt, sink, batch, scale, heads, dim, vdim, out, window=0):
+    """the portions of the step on the matrix cores; k (n_ctx, heads * dim), vt (heads * vdim, n_ctx) from gemm_nt_gather over the rows of
+    batch.context(window); writes its rows of out"""
     _cuda(q, gate, k, vt, sink, out)
     _f32(q, gate, sink)
+    ctx_start, ctx_pos0, _, _ = batch.context(window)
     check(lib().zls_latent_attention_prompt(_p(q), _i(q.shape[1]), _i(q_col0), _p(gate), _i(0 if gate is None else gate.shape[1]), _i(g_col0),
-                                            _p(k), _i(k.stride(0)), _p(vt), _i(vt.stride(0)), _p(sink), _p(batch.ctx_start), batch.ref, _f(scale),
-                                            _i(heads), _i(dim), _i(vdim), _p(out), C.c_int(dt_code(out.dtype)), _stream()),
+                                            _p(k), _i(k.stride(0)), _p(vt), _i(vt.stride(0)), _p(sink), _p(ctx_start), batch.ref, _f(scale),
+                                            _i(heads), _i(dim), _i(vdim), _p(out), C.c_int(dt_code(out.dtype)), _i(window), _p(ctx_pos0), _stream()),
           "latent_attention_prompt")
     return out
 
 
 def latent_attention(q, q_col0, gate, g_col0, w_uk, w_uv, sink, cache, batch, scale, heads, dim, vdim, out=None, single_only=False, mfma=True,
-                     n_splits=None):
+                     n_splits=None, window=0):
     _cuda(q, gate, w_uk, w_uv, sink, cache)
     _f32(q, gate, sink)
     rank = cache.shape[2]
@@ -266,12 +299,14 @@ def latent_attention(q, q_col0, gate, g_col0, w_uk, w_uv, sink, cache, batch, sc
     # enough workgroups to fill the chip (256 CUs, a few per CU), at least 64 keys per split
     groups = batch.n_tok * ((heads + 3) // 4)
     if n_splits is None:
-        n_splits = max(1, min((batch.max_ctx + 63) // 64, (1024 + groups - 1) // groups))
+        span = min(batch.max_ctx, window) if window > 0 else batch.max_ctx
+        n_splits = max(1, min((span + 63) // 64, (1024 + groups - 1) // groups))
     ws = torch.empty(int(lib().zls_latent_attention_workspace_bytes(_i(batch.n_tok), _i(heads), _i(rank), _i(n_splits))) // 4,
                      dtype=torch.float32, device=cache.device)
     check(lib().zls_latent_attention(_p(q), _i(q.shape[1]), _i(q_col0), _p(gate), _i(0 if gate is None else gate.shape[1]), _i(g_col0), _p(w_uk),
                                      _p(w_uv), _p(sink), _p(cache), batch.ref, _f(scale), _i(heads), _i(dim), _i(vdim), _i(rank), _p(out),
-                                     C.c_int(dt_code(cache.dtype)), C.c_int(int(single_only)), _p(ws), _i(n_splits), C.c_int(0 if mfma else 1), _stream()),
+                                     C.c_int(dt_code(cache.dtype)), C.c_int(int(single_only)), _p(ws), _i(n_splits), C.c_int(0 if mfma else 1),
+                                     _i(window), _stream()),
           "latent_attention")
     return out
 
@@ -288,6 +323,25 @@ def conv_silu(proj, col0, w, bias, tail, batch):
                               _stream()), "conv_silu")
     check(lib().zls_conv_tail_update(_p(proj), _i(proj.shape[1]), _i(col0), _p(tail), _i(channels), _i(taps), batch.ref, _stream()),
           "conv_tail_update")
+    return out
+
+
+def short_conv(proj, col0, w, in_bias, tail, batch, act=False, bias=None):
+    """causal convolution over `channels` columns of proj from col0: in_bias joins every input, `bias` the result, act: SiLU; the carried
+    tail moves on (two launches)"""
+    _cuda(proj, w, bias, in_bias, tail)
+    _f32(proj, w, bias, in_bias, tail)
+    channels, taps = w.shape
+    if tail is not None and tuple(tail.shape[1:]) != (taps - 1, channels):
+        raise ZLError("short_conv: tail must be (slots, taps - 1, channels)")
+    for t in (bias, in_bias):
+        if t is not None and t.numel() != channels:
+            raise ZLError("short_conv: one bias per channel")
+    out = torch.empty((batch.n_tok, channels), dtype=torch.float32, device=proj.device)
+    check(lib().zls_short_conv(_p(proj), _i(proj.shape[1]), _i(col0), _p(w), _p(bias), _p(in_bias), C.c_int(int(act)), _p(tail), _i(channels),
+                               _i(taps), batch.ref, _p(out), _stream()), "short_conv")
+    check(lib().zls_short_conv_tail(_p(proj), _i(proj.shape[1]), _i(col0), _p(in_bias), _p(tail), _i(channels), _i(taps), batch.ref, _stream()),
+          "short_conv_tail")
     return out
 
 
@@ -345,11 +399,52 @@ def add_layer_norm(x, y, weight, bias, eps, next_weight=None, next_bias=None, dt
     return h2
 
 
+# ---- weighted RMS norm ------------------------------------------------------------------------------------------------------------------
+def rms_norm(x, weight, eps, dtype, rows=None, around_zero=False):
+    """x / sqrt(mean(x^2) + eps) * weight (around_zero: * (1 + weight)) of the rows `rows` (int32 device; None: all) of fp32 x, in `dtype`"""
+    _cuda(x, weight, rows)
+    _f32(x, weight)
+    if rows is not None and rows.dtype != torch.int32:
+        raise ZLError("rms_norm: rows must be int32")
+    if weight.numel() != x.shape[1]:
+        raise ZLError("rms_norm: one weight per column")
+    n = x.shape[0] if rows is None else rows.numel()
+    out = torch.empty((n, x.shape[1]), dtype=dtype, device=x.device)
+    check(lib().zls_rms_norm(_p(x), _p(rows), _p(weight), _f(1.0 if around_zero else 0.0), _f(eps), _i(n), _i(x.shape[1]), _p(out),
+                             C.c_int(dt_code(dtype)), _stream()), "rms_norm")
+    return out
+
+
+def add_rms_norm(x, y, eps, next_weight=None, dtype=None, around_zero=False):
+    """x += y in place; with next_weight also returns the weighted RMS norm of the new x in `dtype`"""
+    _cuda(x, y, next_weight)
+    _f32(x, y, next_weight)
+    if x.shape != y.shape or (next_weight is not None and next_weight.numel() != x.shape[1]):
+        raise ZLError("add_rms_norm: shape mismatch")
+    h2 = torch.empty(x.shape, dtype=dtype, device=x.device) if next_weight is not None else None
+    check(lib().zls_add_rms_norm(_p(x), _p(y), _f(eps), _i(x.shape[0]), _i(x.shape[1]), _p(next_weight), _f(1.0 if around_zero else 0.0), _p(h2),
+                                 C.c_int(dt_code(dtype) if h2 is not None else BF16), _stream()), "add_rms_norm")
+    return h2
+
+
+def scale_softcap(z, scale, cap):
+    """z <- cap * tanh(z * scale / cap) in place (cap <= 0: z * scale); fp32"""
+    _cuda(z)
+    _f32(z)
+    check(lib().zls_scale_softcap(_p(z), _i(z.numel()), _f(scale), _f(cap), _stream()), "scale_softcap")
+    return z
+
+
 # ---- softmax attention over paged keys and values -------------------------------------------------------------------------------------------
-def rope_norm_store(proj, q_col0, k_col0, v_col0, heads, kv_heads, dim, vdim, qk_freq, rot_dims, v_freq, eps, qk_norm, batch, k_cache, v_cache):
-    """rotate / norm the queries in place in proj; rotate / norm the keys and turn the values into the paged planes (None: queries only)"""
+def rope_norm_store(proj, q_col0, k_col0, v_col0, heads, kv_heads, dim, vdim, qk_freq, rot_dims, v_freq, eps, qk_norm, batch, k_cache, v_cache,
+                    interleaved=False, vmix=None):
+    """rotate / norm the queries in place in proj; rotate / norm the keys and turn the values into the paged planes (None: queries only).
+    interleaved: rotated pairs are neighbours (2i, 2i + 1).  vmix = (src, col0, lam): values <- (1 - lam) values + lam src[t][col0 ..]"""
     _cuda(proj, qk_freq, v_freq, k_cache, v_cache)
     _f32(proj, qk_freq, v_freq)
+    vsrc, vcol, vlam = vmix if vmix is not None else (None, 0, 0.0)
+    if vsrc is not None and (vsrc.dtype != torch.float32 or vsrc.dim() != 2 or vsrc.stride(1) != 1 or vsrc.shape[0] != batch.n_tok):
+        raise ZLError("rope_norm_store: the blended values are fp32 rows, one per token")
     if (qk_freq is not None and qk_freq.numel() != rot_dims // 2) or (v_freq is not None and v_freq.numel() != vdim // 2):
         raise ZLError("rope_norm_store: one frequency per rotated pair")
     if k_cache is not None:
@@ -359,11 +454,13 @@ def rope_norm_store(proj, q_col0, k_col0, v_col0, heads, kv_heads, dim, vdim, qk
             # written transposed, (kv_heads * vdim, page_size): the same bytes of the same plane)
     code = dt_code(k_cache.dtype) if k_cache is not None else F32
     check(lib().zls_rope_norm_store(_p(proj), _i(proj.shape[1]), _i(q_col0), _i(k_col0), _i(v_col0), _i(heads), _i(kv_heads), _i(dim), _i(vdim),
-                                    _p(qk_freq), _i(rot_dims), _p(v_freq), _f(eps), C.c_int(int(qk_norm)), batch.ref, _p(k_cache), _p(v_cache),
+                                    _p(qk_freq), _i(rot_dims), _p(v_freq), _f(eps), C.c_int(int(qk_norm)), C.c_int(int(interleaved)), _p(vsrc),
+                                    _i(0 if vsrc is None else vsrc.stride(0)), _i(vcol), _f(vlam), batch.ref, _p(k_cache), _p(v_cache),
                                     C.c_int(code), _stream()), "rope_norm_store")
 
 
-def window_attention(q, q_col0, k_cache, v_cache, batch, scale, window, heads, kv_heads, dim, vdim, all_kv, mfma=True, n_splits=None):
+def window_attention(q, q_col0, k_cache, v_cache, batch, scale, window, heads, kv_heads, dim, vdim, all_kv, mfma=True, n_splits=None,
+                     keep_first=0):
     """Every query head's softmax weights applied to its own (all_kv False) or every kv head's values.  Returns (acc, ml, n_splits) for
     head_mix_gate: fp32 partial sums (n_tok, heads, n_splits, nv) and their (maximum, weight sum).  bf16 portions run on the matrix cores
     when the sizes allow (mfma=False: everything on the plain kernel); single tokens are split over their window's pages."""
@@ -377,7 +474,8 @@ def window_attention(q, q_col0, k_cache, v_cache, batch, scale, window, heads, k
     plain_tokens = batch.n_single if prompt else batch.n_tok
     # the pages a window can touch, and enough workgroups to fill the chip (256 CUs, a few per CU) when few tokens take the plain kernel
     span = min(batch.max_ctx, window) if window > 0 else batch.max_ctx
-    pages = min((span + ps - 2) // ps + 1, (batch.max_ctx + ps - 1) // ps)
+    keep_first = int(keep_first) if window > 0 else 0                # (keys 0 .. keep_first - 1 stay visible behind the window)
+    pages = min((span + ps - 2) // ps + 1 + (keep_first + ps - 1) // ps, (batch.max_ctx + ps - 1) // ps)
     if n_splits is None:
         n_splits = 1 if plain_tokens == 0 else max(1, min(pages, 1024 // (plain_tokens * heads)))
     n_splits = max(1, min(int(n_splits), pages))
@@ -387,34 +485,40 @@ def window_attention(q, q_col0, k_cache, v_cache, batch, scale, window, heads, k
     code = C.c_int(dt_code(k_cache.dtype))
     if prompt:
         check(lib().zls_window_attention_prompt(_p(q), _i(q.shape[1]), _i(q_col0), _p(k_cache), _p(v_cache), batch.ref, _p(batch.q_tiles),
-                                                _i(batch.n_q_tiles), _f(scale), _i(window), _i(heads), _i(kv_heads), _i(dim), _i(vdim),
+                                                _i(batch.n_q_tiles), _f(scale), _i(window), _i(keep_first), _i(heads), _i(kv_heads), _i(dim), _i(vdim),
                                                 C.c_int(int(all_kv)), _p(acc), _p(ml), _i(n_splits), code, _stream()), "window_attention_prompt")
     if plain_tokens:
-        check(lib().zls_window_attention(_p(q), _i(q.shape[1]), _i(q_col0), _p(k_cache), _p(v_cache), batch.ref, _f(scale), _i(window), _i(heads),
+        check(lib().zls_window_attention(_p(q), _i(q.shape[1]), _i(q_col0), _p(k_cache), _p(v_cache), batch.ref, _f(scale), _i(window), _i(keep_first), _i(heads),
                                          _i(kv_heads), _i(dim), _i(vdim), C.c_int(int(all_kv)), _p(acc), _p(ml), _i(n_splits), _i(per),
                                          C.c_int(int(prompt)), code, _stream()), "window_attention")
     return acc, ml, n_splits
 
 
-def head_mix_gate(acc, ml, n_splits, talk, v_freq, gate, g_col0, batch, heads, kv_heads, vdim, dtype):
-    _cuda(acc, ml, talk, v_freq, gate)
-    _f32(acc, ml, talk, v_freq, gate)
+def head_mix_gate(acc, ml, n_splits, talk, v_freq, gate, g_col0, batch, heads, kv_heads, vdim, dtype, sink=None):
+    _cuda(acc, ml, talk, v_freq, gate, sink)
+    _f32(acc, ml, talk, v_freq, gate, sink)
+    if sink is not None and sink.numel() != heads:
+        raise ZLError("head_mix_gate: one sink per head")
     if talk is not None and tuple(talk.shape) != (heads, heads):
         raise ZLError("head_mix_gate: the mixing matrix is (heads, heads)")
     if acc.numel() != batch.n_tok * heads * n_splits * (kv_heads if talk is not None else 1) * vdim or ml.numel() != batch.n_tok * heads * n_splits * 2:
         raise ZLError("head_mix_gate: acc / ml do not fit")
     out = torch.empty((batch.n_tok, heads * vdim), dtype=dtype, device=acc.device)
     check(lib().zls_head_mix_gate(_p(acc), _p(ml), _i(n_splits), _p(talk), _p(v_freq), _p(gate), _i(0 if gate is None else gate.shape[1]),
-                                  _i(g_col0), batch.ref, _i(heads), _i(kv_heads), _i(vdim), _p(out), C.c_int(dt_code(dtype)), _stream()),
+                                  _i(g_col0), _p(sink), batch.ref, _i(heads), _i(kv_heads), _i(vdim), _p(out), C.c_int(dt_code(dtype)), _stream()),
           "head_mix_gate")
     return out
 
 
 # ---- linear attention with a scalar decay -----------------------------------------------------------------------------------------------------
-def decay_scan(proj, q_col0, k_col0, v_col0, act, decay_h, decay_t, gain_t, norm_col, state, heads, dim, vdim, batch, seg_len=None):
-    """S <- a S + b k v^T, y = S^T q per head over the step's portions; fp32 y (n_tok, heads * (vdim + norm_col))"""
-    _cuda(proj, decay_h, decay_t, gain_t, state)
-    _f32(proj, decay_h, decay_t, gain_t, state)
+def decay_scan(proj, q_col0, k_col0, v_col0, act, decay_h, decay_t, gain_t, norm_col, state, heads, dim, vdim, batch, seg_len=None,
+               decay_v=None):
+    """S <- a S + b k v^T, y = S^T q per head over the step's portions; fp32 y (n_tok, heads * (vdim + norm_col)).  The decay a: a constant
+    per head (decay_h), a number per token and head (decay_t), or a vector per token, one number per key channel (decay_v (n_tok, heads * dim))"""
+    _cuda(proj, decay_h, decay_t, gain_t, state, decay_v)
+    _f32(proj, decay_h, decay_t, gain_t, state, decay_v)
+    if decay_v is not None and tuple(decay_v.shape) != (batch.n_tok, heads * dim):
+        raise ZLError("decay_scan: per-channel decays are (n_tok, heads * dim)")
     P = vdim + (1 if norm_col else 0)
     if tuple(state.shape[1:]) != (heads, dim, P):
         raise ZLError("decay_scan: state must be (slots, heads, dim, vdim + norm_col)")
@@ -429,7 +533,7 @@ def decay_scan(proj, q_col0, k_col0, v_col0, act, decay_h, decay_t, gain_t, norm
                          dtype=torch.float32, device=proj.device)
     check(lib().zls_decay_scan(_p(proj), _i(proj.shape[1]), _i(q_col0), _i(k_col0), _i(v_col0), C.c_int(int(act)), _p(decay_h), _p(decay_t),
                                _p(gain_t), C.c_int(int(norm_col)), _p(state), _i(heads), _i(dim), _i(vdim), batch.ref, _p(y), _p(ws), _i(seg_len),
-                               _stream()), "decay_scan")
+                               _p(decay_v), _stream()), "decay_scan")
     return y
 
 
@@ -443,7 +547,18 @@ def exp_gates(proj, i_col0, f_col0, i_bias, f_bias, cap, m_state, heads, batch):
     return out[0], out[1], out[2]
 
 
-def linear_attn_finish(y, norm_col, q_scale, m_vals, den_eps, heads, vdim, norm_groups, weight, eps, gate, g_col0, dtype):
+def lowrank_decay(proj, u_col0, w2, bias, tau):
+    """sigmoid(w2 u + bias)^(1 / tau) per token: u = `low` fp32 columns of proj from u_col0, w2 (channels, low); fp32 (n_tok, channels)"""
+    _cuda(proj, w2, bias)
+    _f32(proj, bias)
+    channels, low = w2.shape
+    alpha = torch.empty((proj.shape[0], channels), dtype=torch.float32, device=proj.device)
+    check(lib().zls_lowrank_decay(_p(proj), _i(proj.shape[1]), _i(u_col0), _i(low), _p(w2), _p(bias), _f(tau), _i(channels), _i(proj.shape[0]),
+                                  _p(alpha), C.c_int(dt_code(w2.dtype)), _stream()), "lowrank_decay")
+    return alpha
+
+
+def linear_attn_finish(y, norm_col, q_scale, m_vals, den_eps, heads, vdim, norm_groups, weight, eps, gate, g_col0, dtype, gate_act="sigmoid"):
     _cuda(y, m_vals, weight, gate)
     _f32(y, m_vals, weight, gate)
     n_tok = y.shape[0]
@@ -452,7 +567,7 @@ def linear_attn_finish(y, norm_col, q_scale, m_vals, den_eps, heads, vdim, norm_
     out = torch.empty((n_tok, heads * vdim), dtype=dtype, device=y.device)
     check(lib().zls_linear_attn_finish(_p(y), _i(int(norm_col)), _f(q_scale), _p(m_vals), _f(den_eps), _i(heads), _i(vdim), _i(norm_groups),
                                        _p(weight), _f(eps), _p(gate), _i(0 if gate is None else gate.shape[1]), _i(g_col0), _i(n_tok), _p(out),
-                                       C.c_int(dt_code(dtype)), _stream()), "linear_attn_finish")
+                                       C.c_int(dt_code(dtype)), C.c_int(1 if gate_act == "silu" else 0), _stream()), "linear_attn_finish")
     return out
 
 
@@ -461,7 +576,7 @@ MOE_TILE = 64           # rows of an expert's tile in the grouped products; 128 
 MOE_BIG_SHARE = 256
 
 
-def moe_route(logits, correction, groups, keep, top, renorm=False):
+def moe_route(logits, correction, groups, keep, top, renorm=False, score="softmax", group_top=1, renorm_eps=0.0):
     _cuda(logits, correction)
     _f32(logits, correction)
     n_tok, n_out = logits.shape
@@ -469,8 +584,10 @@ def moe_route(logits, correction, groups, keep, top, renorm=False):
         raise ZLError("moe_route: one correction per router output")
     ids = torch.empty((n_tok, top), dtype=torch.int32, device=logits.device)
     weights = torch.empty((n_tok, top), dtype=torch.float32, device=logits.device)
-    check(lib().zls_moe_route(_p(logits), _i(n_tok), _i(n_out), _p(correction), _i(groups), _i(keep), _i(top), C.c_int(int(renorm)), _p(ids),
-                              _p(weights), _stream()), "moe_route")
+    if score not in ("softmax", "sigmoid"):
+        raise ZLError("moe_route: scores are softmax or sigmoid")
+    check(lib().zls_moe_route(_p(logits), _i(n_tok), _i(n_out), _p(correction), _i(groups), _i(keep), _i(top), C.c_int(int(renorm)),
+                              C.c_int(1 if score == "sigmoid" else 0), _i(group_top), _f(renorm_eps), _p(ids), _p(weights), _stream()), "moe_route")
     return ids, weights
 
 
@@ -512,6 +629,20 @@ def silu_mul(gu, dtype):
     rows, two_ff = gu.shape
     out = torch.empty((rows, two_ff // 2), dtype=dtype, device=gu.device)
     check(lib().zls_silu_mul(_p(gu), _i(rows), _i(two_ff // 2), _p(out), C.c_int(dt_code(dtype)), _stream()), "silu_mul")
+    return out
+
+
+ACT_KINDS = {"silu": 0, "gelu_tanh": 1, "swish_clamp": 2}
+
+
+def act_mul(gu, dtype, kind="silu", alpha=1.0, limit=0.0, block=0):
+    """act(gate, up) of fp32 rows [gates | ups] (block 0) or blocks of `block` gates followed by their ups; see ACT_KINDS"""
+    _cuda(gu)
+    _f32(gu)
+    rows, two_ff = gu.shape
+    out = torch.empty((rows, two_ff // 2), dtype=dtype, device=gu.device)
+    check(lib().zls_act_mul(_p(gu), _i(rows), _i(two_ff // 2), C.c_int(ACT_KINDS[kind]), _f(alpha), _f(limit), _i(block), _p(out),
+                            C.c_int(dt_code(dtype)), _stream()), "act_mul")
     return out
 
 
