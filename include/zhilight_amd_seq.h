@@ -269,12 +269,13 @@ int zls_moe_align(const int32_t* ids, int64_t n_slots, int64_t top, int64_t n_ex
                   int32_t* tiles, int64_t max_tiles, int32_t* sorted_exp, zl_stream_t s);
 /* y[p] = x[x_rows[p]] . w[expert of p]^T for every sorted position p: w (n_experts, n, k) in `dtype`, x_rows NULL: x[p]; `tiles` from
  * zls_moe_align with the same tile_m (64 or 128: the workgroup's tile).  gated != 0: n = 2 ff rows per expert, stored as blocks of 16 gate rows followed by their 16 up rows
- * (ff % 16 == 0), and y (.., ff) = silu(gate) * up in out_dtype.  Otherwise y (.., n).
+ * (ff % 16 == 0), and y (.., ff) = act(gate, up) in out_dtype with act / act_alpha / act_limit as zls_act_mul's kind / alpha / limit
+ * (0: silu(gate) * up).  Otherwise y (.., n).
  * row_expert (nullable; sorted_exp of zls_moe_align) with n_rows = the number of sorted positions: the few-rows form -- a wave per (row,
  * output column) streams the weight row once instead of a 64-row tile per expert; the same results up to the order of the fp32 sums. */
 int zls_gemm_nt_grouped(const void* x, int64_t ldx, const int32_t* x_rows, const void* w, const int32_t* tiles, int64_t max_tiles,
                         int64_t tile_m, const int32_t* row_expert, int64_t n_rows, void* y, int64_t ldy, int64_t n, int64_t k, int gated,
-                        int dtype, int out_dtype, zl_stream_t s);
+                        int dtype, int out_dtype, int act, float act_alpha, float act_limit, zl_stream_t s);
 /* out[p][c] = silu(gu[p][c]) * gu[p][ff + c]  for rows 0 .. rows - 1 (gu fp32 (rows, 2 ff)), out in `dtype`. */
 int zls_silu_mul(const float* gu, int64_t rows, int64_t ff, void* out, int dtype, zl_stream_t s);
 /* out[p][c] = act(g, u) of gu fp32 (rows, 2 ff) in `dtype`: kind 0 silu(g) u; 1 gelu_tanh(g) u (tanh form); 2 g' sigmoid(alpha g') (u' + 1)

@@ -224,3 +224,71 @@ def model(cfg, weights, tokens, round_to=None):
     if cap > 0:
         logits = cap * torch.tanh(logits / cap)
     return logits, streams
+
+
+def random_weights(cfg, seed=0, fixed_choice=False, low=8):
+    """every tensor the configuration asks for, bf16-representable values (both serving formats start from the same numbers).
+    fixed_choice: the routers' correction terms lie more than 1 apart, so that they alone order the choice scores (sigmoid scores lie in
+    (0, 1)) and no choice is a close call under a rounded router input; the weights of the chosen experts still follow the scores."""
+    g = torch.Generator().manual_seed(seed)
+    W = cfg["width"]
+    sd = {}
+
+    def mat(name, rows, cols, std=None):
+        sd[name] = (torch.randn(rows, cols, generator=g) * (std if std is not None else cols ** -0.5)).to(torch.bfloat16)
+
+    def vec(name, n, std=0.2, mean=0.0):
+        sd[name] = (mean + std * torch.randn(n, generator=g)).to(torch.bfloat16)
+
+    mat("embed", cfg["vocab"], W, 1.5)
+    mat("head", cfg["vocab"], W)
+    vec("final.norm", W)
+    for i, l in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", l["mixer"]
+        vec(p + "norm1", W)
+        H, d, v = m["heads"], m["dim"], m["vdim"]
+        if l["type"] == "attention":
+            G = m["kv_heads"]
+            for n, rows in (("q", H * d), ("k", G * d), ("v", G * v)):
+                mat(p + "mix." + n, rows, W)
+                vec(p + "mix." + n + ".b", rows, 0.3)
+                if m.get("conv"):
+                    sd[p + "mix." + n + ".conv"] = (torch.randn(rows, m["conv"], generator=g) * 0.6).to(torch.bfloat16)
+            sd[p + "mix.vmix"] = torch.tensor(0.3 + 0.1 * i).to(torch.bfloat16)
+            vec(p + "mix.sink", H, 1.0)
+            mat(p + "mix.o", W, H * v)
+        elif l["type"] == "latent_attention":
+            r, R = m["rot_dim"], m["kv_rank"]
+            mat(p + "mix.q", H * (d + r), W)
+            mat(p + "mix.dkv", R + r, W)
+            vec(p + "mix.dkv.norm", R, 0.2, 1.0)
+            mat(p + "mix.uk", H * d, R)
+            mat(p + "mix.uv", H * v, R)
+            mat(p + "mix.o", W, H * v)
+        else:
+            for n, rows in (("q", H * d), ("k", H * d), ("v", H * v), ("g", H * v), ("a1", low)):
+                mat(p + "mix." + n, rows, W)
+            mat(p + "mix.a2", H * d, low, 1.0)
+            vec(p + "mix.a2.b", H * d, 1.0, 2.0)
+            vec(p + "mix.norm", v, 0.2, 1.0)
+            mat(p + "mix.o", W, H * v)
+        f = l.get("mlp")
+        if f is None:
+            continue
+        vec(p + "norm2", W)
+        if f["kind"] == "dense":
+            mat(p + "mlp.gate", f["ff"], W)
+            mat(p + "mlp.up", f["ff"], W)
+            mat(p + "mlp.down", W, f["ff"])
+        else:
+            E, ff = f["router"]["experts"], f["expert"]["ff"]
+            mat(p + "mlp.router", E, W)
+            if fixed_choice:
+                sd[p + "mlp.correction"] = (torch.randperm(E, generator=g).double() * 1.25).to(torch.bfloat16)
+            else:
+                vec(p + "mlp.correction", E, 0.3)
+            for e in range(E):
+                mat(f"{p}mlp.e{e}.gate", ff, W, 2.0 * W ** -0.5)           # (wide enough that the clamps bite)
+                mat(f"{p}mlp.e{e}.up", ff, W, 2.0 * W ** -0.5)
+                mat(f"{p}mlp.e{e}.down", W, ff)
+    return sd

@@ -172,17 +172,6 @@ __global__ __launch_bounds__(256) void k_silu_mul(const float* __restrict__ gu, 
     for (int c = threadIdx.x; c < ff; c += 256) SeqT<DT>::st(out, r * ff + c, seq_silu(gu[r * 2 * ff + c]) * gu[r * 2 * ff + ff + c]);
 }
 
-// kind 0: silu(g) u; 1: gelu_tanh(g) u; 2: g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit)
-__device__ __forceinline__ float gated_act(float g, float u, int kind, float alpha, float limit) {
-    if (kind == 1) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
-    if (kind == 2) {
-        g = fminf(g, limit);
-        u = fminf(fmaxf(u, -limit), limit);
-        return g * seq_sigmoid(alpha * g) * (u + 1.0f);
-    }
-    return seq_silu(g) * u;
-}
-
 // block > 0: the row holds blocks of `block` gate columns followed by their `block` up columns; 0: all gates, then all ups
 template <int DT>
 __global__ __launch_bounds__(256) void k_act_mul(const float* __restrict__ gu, int ff, int kind, float alpha, float limit, int block,

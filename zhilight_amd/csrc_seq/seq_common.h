@@ -19,6 +19,17 @@ template <> struct SeqT<ZL_F32> {
 __device__ __forceinline__ float seq_silu(float v) { return v / (1.0f + expf(-v)); }
 __device__ __forceinline__ float seq_sigmoid(float v) { return 1.0f / (1.0f + expf(-v)); }
 __device__ __forceinline__ float seq_softplus(float v) { return v > 20.0f ? v : log1pf(expf(v)); }
+// the gated activations of the feed-forwards
+// kind 0: silu(g) u; 1: gelu_tanh(g) u; 2: g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit)
+__device__ __forceinline__ float gated_act(float g, float u, int kind, float alpha, float limit) {
+    if (kind == 1) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+    if (kind == 2) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        return g * seq_sigmoid(alpha * g) * (u + 1.0f);
+    }
+    return seq_silu(g) * u;
+}
 // sine and cosine of an fp32 angle of any size (positions times frequencies reach thousands of radians): the angle is brought into
 // [-pi, pi] in double (exact to 1e-9 for angles up to 2^24), where the fp32 functions take their short path
 __device__ __forceinline__ void seq_sincos(float a, float* sn, float* cs) {

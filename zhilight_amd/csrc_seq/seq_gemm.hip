@@ -28,6 +28,7 @@ struct GemmP {
     // the expert-sorted order, w = the expert's (n, k) block of a stacked (experts, n, k) array; expert < 0: the tile is unused
     const int32_t* tiles;
     int64_t w_stride;
+    int act; float act_alpha, act_limit;                       // the gated epilogue's activation (gated_act in seq_common.h)
 };
 
 // ---- tiles in LDS -----------------------------------------------------------------------------------------------------------------
@@ -71,7 +72,7 @@ template <> struct Tile<ZL_F32> {
 
 // WT x WT MFMA tiles per wave: the workgroup's output tile is (32 WT) x (32 WT)
 // GATED: the weight rows come in blocks of 16 gate rows followed by their 16 up rows, so that a wave's even column tiles are gates and the
-// odd ones the up projections of the same 16 outputs; the epilogue writes silu(gate) * up, half as many columns
+// odd ones the up projections of the same 16 outputs; the epilogue writes act(gate, up) (gated_act: silu(gate) * up and others), half as many columns
 template <int DT, int ODT, int WT, bool GATED = false>
 __global__ __launch_bounds__(256) void k_seq_gemm(const GemmP p) {
     typedef typename Tile<DT>::elem E;
@@ -166,7 +167,7 @@ __global__ __launch_bounds__(256) void k_seq_gemm(const GemmP p) {
                 for (int r = 0; r < 4; ++r) {
                     const int row = m0 + wm * 16 * WT + i * 16 + 4 * kq + r;
                     if (row < mlim && wcol < p.n)
-                        SeqT<ODT>::st(p.y, (size_t)row * p.ldy + col, seq_silu(acc[i][2 * jj][r]) * acc[i][2 * jj + 1][r]);
+                        SeqT<ODT>::st(p.y, (size_t)row * p.ldy + col, gated_act(acc[i][2 * jj][r], acc[i][2 * jj + 1][r], p.act, p.act_alpha, p.act_limit));
                 }
         }
         return;
@@ -299,7 +300,7 @@ __global__ __launch_bounds__(256) void k_seq_gemv_mfma(const GemmP p) {
 
 // the grouped product for a FEW rows (decode steps of a mixture of experts): a wave per (sorted row, output column) streams the column's
 // weight row of the row's expert once, 16-byte loads -- a 64-row tile per expert would multiply 63 rows of zeros and leave most of the
-// chip idle.  GATED: the gate row and its up row (16 rows further in the packed block), silu(gate) * up.
+// chip idle.  GATED: the gate row and its up row (16 rows further in the packed block), act(gate, up).
 template <int DT, int ODT, bool GATED>
 __global__ __launch_bounds__(256) void k_seq_gemv_grouped(const GemmP p, const int32_t* __restrict__ row_expert, int n_rows) {
     const int lane = threadIdx.x & 63;
@@ -333,7 +334,7 @@ __global__ __launch_bounds__(256) void k_seq_gemv_grouped(const GemmP p, const i
         }
     }
     a0 = zl_wave_sum(a0);
-    if constexpr (GATED) a0 = seq_silu(a0) * zl_wave_sum(a1);
+    if constexpr (GATED) a0 = gated_act(a0, zl_wave_sum(a1), p.act, p.act_alpha, p.act_limit);
     if (lane == 0) SeqT<ODT>::st(p.y, (size_t)row * p.ldy + col, a0);
 }
 
@@ -379,7 +380,7 @@ extern "C" int zls_gemm_nt(const void* x, int64_t ldx, const void* w, void* y, i
     ZL_CHECK_ARG((m + 63) / 64 <= 65535, ZL_ELIMIT);
     ZL_CHECK_ARG(dtype == ZL_BF16 || dtype == ZL_F32, ZL_EDTYPE);
     ZL_CHECK_ARG(out_dtype == ZL_F32 || out_dtype == dtype, ZL_EDTYPE);
-    GemmP p;
+    GemmP p = {};
     p.x = x; p.w = w; p.y = y; p.ldx = ldx; p.ldw = k; p.ldy = ldy; p.m = (int)m; p.n = (int)n; p.k = (int)k;
     p.x_rows = p.w_rows = nullptr; p.tiles = nullptr; p.w_stride = 0;
     const int64_t unit = dtype == ZL_BF16 ? 8 : 4;
@@ -398,7 +399,7 @@ extern "C" int zls_gemm_nt_gather(const void* x, int64_t ldx, const int32_t* x_r
     ZL_CHECK_ARG((m + 63) / 64 <= 65535, ZL_ELIMIT);
     ZL_CHECK_ARG(dtype == ZL_BF16 || dtype == ZL_F32, ZL_EDTYPE);
     ZL_CHECK_ARG(out_dtype == ZL_F32 || out_dtype == dtype, ZL_EDTYPE);
-    GemmP p;
+    GemmP p = {};
     p.x = x; p.w = w; p.y = y; p.ldx = ldx; p.ldw = ldw; p.ldy = ldy; p.m = (int)m; p.n = (int)n; p.k = (int)k;
     p.x_rows = x_rows; p.w_rows = w_rows; p.tiles = nullptr; p.w_stride = 0;
     const int64_t unit = dtype == ZL_BF16 ? 8 : 4;
@@ -418,7 +419,8 @@ extern "C" int zls_gemm_nt_gather(const void* x, int64_t ldx, const int32_t* x_r
 // caller aligns with the same size: 128 when the experts' shares are long enough to fill them).
 extern "C" int zls_gemm_nt_grouped(const void* x, int64_t ldx, const int32_t* x_rows, const void* w, const int32_t* tiles, int64_t max_tiles,
                                    int64_t tile_m, const int32_t* row_expert, int64_t n_rows, void* y, int64_t ldy, int64_t n, int64_t k, int gated,
-                                   int dtype, int out_dtype, zl_stream_t s) {
+                                   int dtype, int out_dtype, int act, float act_alpha, float act_limit, zl_stream_t s) {
+    ZL_CHECK_ARG(act >= 0 && act <= 2, ZL_EINVAL);
     ZL_CHECK_ARG(x && w && tiles && y && max_tiles > 0 && n > 0 && k > 0, ZL_EINVAL);
     ZL_CHECK_ARG(tile_m == 64 || tile_m == 128, ZL_ESHAPE);
     ZL_CHECK_ARG(!row_expert || (n_rows > 0 && n_rows <= 65535), ZL_ESHAPE);
@@ -426,9 +428,10 @@ extern "C" int zls_gemm_nt_grouped(const void* x, int64_t ldx, const int32_t* x_
     ZL_CHECK_ARG(dtype == ZL_BF16 || dtype == ZL_F32, ZL_EDTYPE);
     ZL_CHECK_ARG(out_dtype == ZL_F32 || out_dtype == dtype, ZL_EDTYPE);
     ZL_CHECK_ARG(gated ? (n % 32 == 0 && ldy >= n / 2) : ldy >= n, ZL_ESHAPE);
-    GemmP p;
+    GemmP p = {};
     p.x = x; p.w = w; p.y = y; p.ldx = ldx; p.ldw = k; p.ldy = ldy; p.m = 0; p.n = (int)n; p.k = (int)k;
     p.x_rows = x_rows; p.w_rows = nullptr; p.tiles = tiles; p.w_stride = n * k;
+    p.act = act; p.act_alpha = act_alpha; p.act_limit = act_limit;
     const int64_t unit = dtype == ZL_BF16 ? 8 : 4;
     p.vec = (k % unit == 0 && ldx % unit == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) ? 1 : 0;
     hipStream_t hs = (hipStream_t)s;

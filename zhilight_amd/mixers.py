@@ -538,7 +538,7 @@ class RoutedExpertsFF:
         self.width, self.ff, self.experts, self.top, self.identity = width, ff, experts, top, identity
         self.groups, self.keep, self.has_correction, self.renorm = groups, keep, correction, renorm
         self.packed = ff % 16 == 0                       # gate / up rows in blocks of 16: what the gated epilogue reads
-        self.fused_act = self.packed and act == "silu"   # (the products' epilogue knows silu(gate) * up; other activations take one more launch)
+        self.fused_act = self.packed                     # (the grouped product's epilogue finishes the activation)
         self.few_rows = seqops.MOE_FEW_ROWS
         self.tile_m = None                # rows per expert tile of the grouped products (None: by the experts' average share)
 
@@ -579,7 +579,8 @@ class RoutedExpertsFF:
         n_slots = ids.numel()
         few = sorted_exp if n_slots <= self.few_rows else None                    # decode steps: weight rows streamed per (row, column)
         if self.fused_act:
-            a = seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots, gated=True, out_dtype=h.dtype, row_expert=few, tile_m=tm)
+            a = seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots, gated=True, out_dtype=h.dtype, row_expert=few, tile_m=tm,
+                                       act=self.act, act_alpha=self.act_alpha, act_limit=self.limit)
         else:
             a = seqops.act_mul(seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots, row_expert=few, tile_m=tm), h.dtype,
                                kind=self.act, alpha=self.act_alpha, limit=self.limit, block=16 if self.packed else 0)

@@ -609,9 +609,13 @@ def moe_align(ids, n_experts, tile_m=None):
     return sorted_tok, slot_pos, tiles, max_tiles, sorted_exp, tile_m
 
 
-def gemm_nt_grouped(x, x_rows, w, tiles, max_tiles, n_rows, gated=False, out_dtype=torch.float32, row_expert=None, tile_m=MOE_TILE):
+ACT_KINDS = {"silu": 0, "gelu_tanh": 1, "swish_clamp": 2}
+
+
+def gemm_nt_grouped(x, x_rows, w, tiles, max_tiles, n_rows, gated=False, out_dtype=torch.float32, row_expert=None, tile_m=MOE_TILE,
+                    act="silu", act_alpha=1.0, act_limit=0.0):
     """rows of x (gathered by x_rows, or in sorted order) times their expert's block of w (experts, n, k); (n_rows, n or n / 2 gated).
-    row_expert (the sorted positions' experts) selects the few-rows kernel."""
+    row_expert (the sorted positions' experts) selects the few-rows kernel.  act (ACT_KINDS) is the gated form's activation."""
     _cuda(x, x_rows, w, tiles, row_expert)
     E, n, k = w.shape
     if x.shape[1] != k or x.dtype != w.dtype:
@@ -619,7 +623,7 @@ def gemm_nt_grouped(x, x_rows, w, tiles, max_tiles, n_rows, gated=False, out_dty
     out = torch.empty((n_rows, n // 2 if gated else n), dtype=out_dtype, device=x.device)
     check(lib().zls_gemm_nt_grouped(_p(x), _i(x.stride(0)), _p(x_rows), _p(w), _p(tiles), _i(max_tiles), _i(tile_m), _p(row_expert), _i(n_rows), _p(out),
                                     _i(out.shape[1]), _i(n), _i(k), C.c_int(int(gated)), C.c_int(dt_code(x.dtype)), C.c_int(dt_code(out_dtype)),
-                                    _stream()), "gemm_nt_grouped")
+                                    C.c_int(ACT_KINDS[act]), _f(act_alpha), _f(act_limit), _stream()), "gemm_nt_grouped")
     return out
 
 
@@ -630,9 +634,6 @@ def silu_mul(gu, dtype):
     out = torch.empty((rows, two_ff // 2), dtype=dtype, device=gu.device)
     check(lib().zls_silu_mul(_p(gu), _i(rows), _i(two_ff // 2), _p(out), C.c_int(dt_code(dtype)), _stream()), "silu_mul")
     return out
-
-
-ACT_KINDS = {"silu": 0, "gelu_tanh": 1, "swish_clamp": 2}
 
 
 def act_mul(gu, dtype, kind="silu", alpha=1.0, limit=0.0, block=0):
