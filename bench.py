@@ -18,10 +18,12 @@ fields, `roofline` (the W4A16 GEMV kernel: algorithmic bytes / HIP-event time, v
 
     python bench.py --mixers 1b,8b [--seq 2048]
     python bench.py --retotar 1b,8b [--seq 2048]
+    python bench.py --gutivik 1b,8b [--seq 2048]
 
 is a different measurement with its own JSON line: prefill / decode throughput of the ragged-step engine's latent-attention, state-space
 and hybrid stacks (zhilight_amd/tupitar.py) beside the dense bf16 Llama-shaped stack of equal width, 4 layers each, random weights;
 --retotar the same for the Retotar stacks (zhilight_amd/retotar.py) beside the Tupitar hybrid of equal width.
+--gutivik the same for the Gutivik stacks (zhilight_amd/gutivik.py) beside Retotar stacks of equal width.
 """
 import argparse
 import json
@@ -600,11 +602,101 @@ def bench_retotar(args, dev):
     print(json.dumps({"metric": "retotar_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "layers": 4, "results": results}))
 
 
+GUTIVIK_BENCH_SIZES = {
+    # name: width; attention heads / key-value heads x head size, window, kept first tokens, taps, rotated part; latent attention heads x
+    #       (plain + rotated) key size, latent rank; gated-linear-attention heads x key size x value size, rank of the decay's projection pair;
+    #       experts x their ff, picks, groups.  Head counts, windows and experts are those of RETOTAR_BENCH_SIZES, so the stacks beside them
+    #       move the same weights per token.
+    "1b": dict(width=2048, heads=16, kv_heads=4, dim=128, window=1024, keep=4, taps=4, rot=64, l_dim=128, l_rot=64, rank=512,
+               g_heads=16, g_dim=128, g_vdim=128, low=16, experts=16, ff=1360, top=4, groups=4, keep_groups=2),
+    "8b": dict(width=4096, heads=32, kv_heads=8, dim=128, window=1024, keep=4, taps=4, rot=64, l_dim=128, l_rot=64, rank=512,
+               g_heads=32, g_dim=128, g_vdim=128, low=16, experts=32, ff=2384, top=4, groups=4, keep_groups=2),
+}
+
+
+def bench_gutivik(args, dev):
+    """--gutivik: prefill and decode throughput of Gutivik stacks (zhilight_amd/gutivik.py: attention with a short convolution, kept first
+    keys, sink and blended values; latent attention with a rotated key part and a window; gated linear attention with a decay per key
+    channel; sigmoid-routed experts) beside the closest existing model of equal width, Retotar (windowed attention, linear attention with
+    a scalar decay, softmax-routed experts), 4 layers each, random weights, bf16, eager launches.  One JSON line."""
+    from zhilight_amd.engine import Engine, Entry
+    from zhilight_amd.gutivik import GutivikConfig, GutivikLayerConfig, GutivikModel
+    from zhilight_amd.retotar import RetotarConfig, RetotarLayerConfig, RetotarModel
+    seq, vocab, results = args.seq, 32000, []
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    def measure(label, name, model):
+        toks = torch.randint(0, vocab, (seq,)).tolist()
+        for batch in (1, 8):
+            eng = Engine(model, max_tokens=batch * (seq + 64), max_seqs=batch)
+
+            def prefill():
+                eng.run_step([Entry("p", toks, [seq - 1])])
+                eng.release("p")
+            if batch == 1:
+                ms = timed(prefill, 3)
+                results.append(dict(model=label, size=name, phase="prefill", tokens=seq, ms=round(ms, 3), tokens_per_s=round(seq / ms * 1e3)))
+            for b in range(batch):
+                eng.run_step([Entry(f"d{b}", toks[:seq - 40], [])])
+
+            def decode():
+                eng.run_step([Entry(f"d{b}", [7], [0]) for b in range(batch)])
+            ms = timed(decode, 20)
+            results.append(dict(model=label, size=name, phase="decode", batch=batch, context=seq - 40, ms=round(ms, 3),
+                                tokens_per_s=round(batch / ms * 1e3)))
+            del eng
+
+    for name in args.gutivik.split(","):
+        z = GUTIVIK_BENCH_SIZES[name]
+        mlp = dict(kind="moe", expert=dict(ff=z["ff"], limit=7.0), router=dict(experts=z["experts"], top=z["top"],
+                                                                               groups=dict(count=z["groups"], keep=z["keep_groups"])))
+        att = dict(heads=z["heads"], kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["dim"], scale=z["dim"] ** -0.5, conv=z["taps"],
+                   mask=dict(size=z["window"], keep_first=z["keep"]), rot=dict(dims=z["rot"], base=5e5), v_mix=True)
+        lat = dict(heads=z["heads"], dim=z["l_dim"], rot_dim=z["l_rot"], vdim=z["dim"], kv_rank=z["rank"], scale=(z["l_dim"] + z["l_rot"]) ** -0.5,
+                   mask=dict(size=z["window"]), rot=dict(dims=z["l_rot"], base=1e4))
+        gla = dict(heads=z["g_heads"], dim=z["g_dim"], vdim=z["g_vdim"], tau=16.0)
+        A, L, G = (GutivikLayerConfig(t, m, mlp) for t, m in (("attention", att), ("latent_attention", lat), ("gla", gla)))
+        for label, layers in (("attention x4", [A] * 4), ("latent_attention x4", [L] * 4), ("gla x4", [G] * 4), ("hybrid (a, l, g, a)", [A, L, G, A])):
+            model = GutivikModel(GutivikConfig(vocab, z["width"], 1e-6, 0.25, 30.0, 1 << 24, layers), "bfloat16", dev).init_random(1)
+            measure("gutivik " + label, name, model)
+            del model
+        r = RETOTAR_BENCH_SIZES[name]
+        total = r["experts"] + r["identity"]
+        rmlp = dict(kind="moe", expert=dict(ff=r["ff"]), router=dict(experts=r["experts"], identity=r["identity"], top=r["top"],
+                                                                     groups=dict(count=r["groups"] if total % r["groups"] == 0 else 1, keep=r["keep"])))
+        if rmlp["router"]["groups"]["count"] == 1:
+            rmlp["router"]["groups"]["keep"] = 1
+        ratt = dict(heads=r["heads"], kv_heads=r["kv_heads"], dim=r["dim"], vdim=r["dim"], scale=r["dim"] ** -0.5, mask=dict(size=r["window"]),
+                    rot=dict(dims=r["rot"], base=1e6, scaling=dict(factor=1.0)))
+        rlin = dict(heads=r["l_heads"], dim=r["l_dim"], vdim=r["l_vdim"], decay=[1.0 - 2.0 ** -(3 + 5 * h / r["l_heads"]) for h in range(r["l_heads"])])
+        RA = lambda **kw: RetotarLayerConfig("attention", dict(ratt, **kw), rmlp)
+        RL = RetotarLayerConfig("lightning", rlin, rmlp)
+        for label, layers in (("attention x4", [RA(), RA(kv_from=0), RA(), RA(kv_from=2)]), ("lightning x4", [RL] * 4),
+                              ("hybrid (a, l, l, a)", [RA(), RL, RL, RA()])):
+            model = RetotarModel(RetotarConfig(vocab, r["width"], 1.0, 1e-6, 1 << 24, layers), "bfloat16", dev).init_random(1)
+            measure("retotar " + label, name, model)
+            del model
+    print(json.dumps({"metric": "gutivik_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "layers": 4, "results": results}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--retotar", default="", metavar="SIZES",
                     help="instead of the default workload: prefill / decode throughput of Retotar stacks beside the Tupitar hybrid of equal "
                          "width; comma-separated sizes of " + ", ".join(RETOTAR_BENCH_SIZES))
+    ap.add_argument("--gutivik", default="", metavar="SIZES",
+                    help="instead of the default workload: prefill / decode throughput of Gutivik stacks beside Retotar stacks of equal "
+                         "width; comma-separated sizes of " + ", ".join(GUTIVIK_BENCH_SIZES))
     ap.add_argument("--mixers", default="", metavar="SIZES",
                     help="instead of the default workload: prefill / decode throughput of the ragged-step engine's latent-attention + "
                          "state-space model beside the dense Llama-shaped stack of equal width; comma-separated sizes of " + ", ".join(SEQ_BENCH_SIZES))
@@ -646,6 +738,8 @@ def main():
         return bench_sequence_mixers(args, dev)
     if args.retotar:
         return bench_retotar(args, dev)
+    if args.gutivik:
+        return bench_gutivik(args, dev)
     from zhilight_amd import ops  # noqa: F401  (raises if the HIP library is missing)
     from zhilight_amd.llama import LLaMA, ModelConfig, QuantConfig
 

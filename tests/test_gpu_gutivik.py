@@ -374,6 +374,21 @@ def test_latent_attention_rotated_part_and_window_edges(dev, dtype, window):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_latent_attention_with_a_wide_latent(dev, dtype):
+    """a cached row of 512 + 64 numbers (another instantiation of the single-token kernel), heads of 64 + 64"""
+    layer = latent_cfg(heads=3, dim=64, rot=64, vdim=48, rank=512, size=90, scale=0.09)
+    W, T = 128, 200
+    cfg = model_cfg([layer], width=W)
+    sd = O.random_weights(cfg, 9)
+    h = bf(torch.randn(T, W, generator=torch.Generator().manual_seed(10)))
+    ref = O.latent_attention_mixer(h, sd, "l0.mix.", layer["mixer"], EPS)
+    cache = new_cache(dev)
+    mix = build_mixer(layer, sd, "l0.mix.", W, dtype, dev, cache)
+    cache.admit("s")
+    assert_close(feed(mix, cache, h.to(dtype), [120] + [1] * 20 + [60], dev), ref, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,dim,vdim,tau", [(2, 40, 24, 8.0), (1, 70, 9, 1.0), (3, 16, 64, 16.0), (2, 128, 128, 4.0)])
 def test_gated_linear_attention_in_portions_and_segments(dev, dtype, heads, dim, vdim, tau):
     layer = gla_cfg(heads, dim, vdim, tau)

@@ -634,14 +634,16 @@ extern "C" int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0,
     p.heads = (int)heads; p.dim = (int)dim; p.vdim = (int)vdim; p.rank = (int)rank; p.scale = scale; p.single_only = single_only;
     ZL_CHECK_ARG(window < (1 << 30), ZL_ESHAPE);
     p.window = window > 0 ? (int)window : 0;
-    p.vec = (rank % (dtype == ZL_BF16 ? 8 : 4) == 0 && ((uintptr_t)cache & 15) == 0) ? 1 : 0;
+    // (the split kernel's eight 16-byte slots per thread cover 1024 bf16 or 512 fp32 columns of a row; longer fp32 rows are read singly)
+    p.vec = (rank % (dtype == ZL_BF16 ? 8 : 4) == 0 && ((uintptr_t)cache & 15) == 0 && (dtype == ZL_BF16 || rank <= 512)) ? 1 : 0;
     const dim3 grid(b->n_tok, (unsigned)((heads + 3) / 4), (unsigned)n_splits);
     hipStream_t hs = (hipStream_t)s;
     float* ws = (float*)workspace;
     float* qa = ws + (size_t)b->n_tok * heads * n_splits * (rank + 2);
     const int ns = (int)n_splits;
-    // bf16 with aligned rows of at most 512 latent columns: the split pass on the matrix cores (absorb and combine are shared)
-    const bool mfma = dtype == ZL_BF16 && p.vec && rank <= 512 && !no_mfma;
+    // bf16 with aligned rows of at most 640 latent columns (512 + a rotated part): the split pass on the matrix cores (absorb and combine
+    // are shared)
+    const bool mfma = dtype == ZL_BF16 && p.vec && rank <= 640 && !no_mfma;
     const dim3 mgrid(b->n_tok, (unsigned)((heads + 15) / 16), (unsigned)n_splits);
 #define MSPLIT(RT) hipLaunchKernelGGL((k_latent_decode_mfma<RT>), mgrid, dim3(64), 0, hs, p, *b, qa, ws, ns)
 #define SPLIT(DT, RPL) hipLaunchKernelGGL((k_latent_split<DT, RPL>), grid, dim3(256), lds, hs, p, *b, qa, ws, ns)
@@ -651,7 +653,8 @@ extern "C" int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0,
         if (rank <= 64) MSPLIT(2);                \
         else if (rank <= 128) MSPLIT(4);          \
         else if (rank <= 256) MSPLIT(8);          \
-        else MSPLIT(16);                          \
+        else if (rank <= 512) MSPLIT(16);         \
+        else MSPLIT(20);                          \
     } else if (rank <= 64) SPLIT(DT, 1);          \
     else if (rank <= 128) SPLIT(DT, 2);           \
     else if (rank <= 256) SPLIT(DT, 4);           \
