@@ -667,6 +667,8 @@ def bench_gutivik(args, dev):
         gla = dict(heads=z["g_heads"], dim=z["g_dim"], vdim=z["g_vdim"], tau=16.0)
         A, L, G = (GutivikLayerConfig(t, m, mlp) for t, m in (("attention", att), ("latent_attention", lat), ("gla", gla)))
         for label, layers in (("attention x4", [A] * 4), ("latent_attention x4", [L] * 4), ("gla x4", [G] * 4), ("hybrid (a, l, g, a)", [A, L, G, A])):
+            if args.only and args.only not in "gutivik " + label:
+                continue
             model = GutivikModel(GutivikConfig(vocab, z["width"], 1e-6, 0.25, 30.0, 1 << 24, layers), "bfloat16", dev).init_random(1)
             measure("gutivik " + label, name, model)
             del model
@@ -683,6 +685,8 @@ def bench_gutivik(args, dev):
         RL = RetotarLayerConfig("lightning", rlin, rmlp)
         for label, layers in (("attention x4", [RA(), RA(kv_from=0), RA(), RA(kv_from=2)]), ("lightning x4", [RL] * 4),
                               ("hybrid (a, l, l, a)", [RA(), RL, RL, RA()])):
+            if args.only and args.only not in "retotar " + label:
+                continue
             model = RetotarModel(RetotarConfig(vocab, r["width"], 1.0, 1e-6, 1 << 24, layers), "bfloat16", dev).init_random(1)
             measure("retotar " + label, name, model)
             del model
@@ -697,6 +701,7 @@ def main():
     ap.add_argument("--gutivik", default="", metavar="SIZES",
                     help="instead of the default workload: prefill / decode throughput of Gutivik stacks beside Retotar stacks of equal "
                          "width; comma-separated sizes of " + ", ".join(GUTIVIK_BENCH_SIZES))
+    ap.add_argument("--only", default="", metavar="TEXT", help="with --gutivik: only the stacks whose label contains TEXT (e.g. for a kernel trace of one model)")
     ap.add_argument("--mixers", default="", metavar="SIZES",
                     help="instead of the default workload: prefill / decode throughput of the ragged-step engine's latent-attention + "
                          "state-space model beside the dense Llama-shaped stack of equal width; comma-separated sizes of " + ", ".join(SEQ_BENCH_SIZES))

@@ -684,11 +684,11 @@ extern "C" int zls_latent_attention_prompt(const float* q, int64_t ldq, int64_t 
     p.tiles_per_seq = (b->max_count + 63) / 64;
     p.vec_k = (dim % 8 == 0 && ldk % 8 == 0 && ((uintptr_t)k & 15) == 0) ? 1 : 0;
     const dim3 grid((unsigned)(b->n_seq * p.tiles_per_seq), (unsigned)heads);
-    const int64_t big = dim > vdim ? dim : vdim;
     hipStream_t hs = (hipStream_t)s;
-    if (big <= 32) hipLaunchKernelGGL((k_latent_fa<1, 2>), grid, dim3(256), 0, hs, p, *b);
-    else if (big <= 64) hipLaunchKernelGGL((k_latent_fa<2, 4>), grid, dim3(256), 0, hs, p, *b);
-    else if (big <= 128) hipLaunchKernelGGL((k_latent_fa<4, 8>), grid, dim3(256), 0, hs, p, *b);
-    else hipLaunchKernelGGL((k_latent_fa<8, 16>), grid, dim3(256), 0, hs, p, *b);
-    return zl_launch_status();
+    // the smallest instantiation that holds both the key size (32 DK) and the value size (16 DV): heads with a rotated part have keys
+    // longer than their values
+#define FA(DK, DV) if (dim <= 32 * DK && vdim <= 16 * DV) { hipLaunchKernelGGL((k_latent_fa<DK, DV>), grid, dim3(256), 0, hs, p, *b); return zl_launch_status(); }
+    FA(1, 2) FA(2, 2) FA(2, 4) FA(4, 4) FA(4, 8) FA(6, 8) FA(8, 8) FA(8, 16)
+#undef FA
+    return ZL_ESHAPE;
 }

@@ -94,10 +94,10 @@ __global__ __launch_bounds__(kG) void k_linear_attn_finish(const FinP p) {
         return v;
     };
     float ss = 0.f;
-    for (int i = threadIdx.x; i < p.part; i += kG) { const float v = value(c0 + i); ss = fmaf(v, v, ss); }
+    for (int i = threadIdx.x; i < p.part; i += blockDim.x) { const float v = value(c0 + i); ss = fmaf(v, v, ss); }
     ss = zl_block_sum(ss, red);
     const float f = 1.0f / sqrtf(ss / (float)p.part + p.eps);
-    for (int i = threadIdx.x; i < p.part; i += kG) {
+    for (int i = threadIdx.x; i < p.part; i += blockDim.x) {
         const int c = c0 + i;
         float v = value(c) * f;
         if (p.weight) v *= p.weight[c];
@@ -129,7 +129,9 @@ extern "C" int zls_linear_attn_finish(const float* y, int64_t norm_col, float q_
     p.y = y; p.m_vals = m_vals; p.weight = weight; p.gate = gate; p.ldg = ldg; p.norm_col = norm_col ? 1 : 0; p.heads = (int)heads;
     p.vdim = (int)vdim; p.part = (int)(heads * vdim / norm_groups); p.g_col0 = (int)g_col0; p.q_scale = q_scale; p.den_eps = den_eps;
     p.eps = eps; p.out = out; p.gate_kind = gate_kind == 1 ? 1 : 0;
-#define CALL(DT) hipLaunchKernelGGL((k_linear_attn_finish<DT>), dim3((unsigned)n_tok, (unsigned)norm_groups), dim3(kG), 0, (hipStream_t)s, p);
+    // (a norm group per workgroup: short groups -- a head each -- get no more waves than they have elements for)
+    const unsigned threads = p.part >= kG ? kG : (unsigned)((p.part + 63) / 64 * 64);
+#define CALL(DT) hipLaunchKernelGGL((k_linear_attn_finish<DT>), dim3((unsigned)n_tok, (unsigned)norm_groups), dim3(threads), 0, (hipStream_t)s, p);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
     return zl_launch_status();
