@@ -218,18 +218,33 @@ __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batc
     if (p.mode == 1 && tid == 0 && !p.vec) p.seg_prod[seg_at] = prod;
 }
 
-// vector decays: the product of a segment's decays per (sequence, segment, head, state row), tokens in order; the last segment needs none
-__global__ __launch_bounds__(256) void k_seg_decay_prod(const ScanP p, const zls_batch_t b) {
+// vector decays: the product of a segment's decays per (sequence, segment, head, state row); the last segment needs none.  The 1024 threads
+// are (row, part of the segment's tokens): every part multiplies its tokens in order, the parts meet in LDS and are multiplied in order
+__global__ __launch_bounds__(1024) void k_seg_decay_prod(const ScanP p, const zls_batch_t b) {
+    __shared__ float part[1024];
     const int sq = blockIdx.x / p.n_seg, seg = blockIdx.x % p.n_seg, h = blockIdx.y, N = p.n_state;
     const int whole = b.seq_start[sq + 1] - b.seq_start[sq];
     if ((seg + 1) * p.seg_len >= whole) return;
     const int first = b.seq_start[sq] + seg * p.seg_len;
     const size_t seg_at = ((size_t)sq * p.n_seg + seg) * p.heads + h;
-    for (int n = threadIdx.x; n < N; n += 256) {
+    int rows = 1;
+    while (rows < N && rows < 1024) rows <<= 1;                           // rows per pass (a power of two), 1024 / rows parts
+    const int parts = 1024 / rows, r = threadIdx.x % rows, j = threadIdx.x / rows;
+    const int per = (p.seg_len + parts - 1) / parts, t0 = j * per, t1 = min(p.seg_len, t0 + per);
+    for (int n0 = 0; n0 < N; n0 += rows) {
+        const int n = n0 + r;
         float prod = 1.0f;
-        const float* a = p.decay_v + (size_t)first * p.heads * N + (size_t)h * N + n;
-        for (int i = 0; i < p.seg_len; ++i) prod *= a[(size_t)i * p.heads * N];
-        p.seg_prod[seg_at * N + n] = prod;
+        if (n < N) {
+            const float* a = p.decay_v + (size_t)first * p.heads * N + (size_t)h * N + n;
+            for (int i = t0; i < t1; ++i) prod *= a[(size_t)i * p.heads * N];
+        }
+        part[threadIdx.x] = prod;
+        __syncthreads();
+        if (j == 0 && n < N) {
+            for (int q = 1; q < parts; ++q) prod *= part[q * rows + r];
+            p.seg_prod[seg_at * N + n] = prod;
+        }
+        __syncthreads();
     }
 }
 
@@ -358,7 +373,7 @@ static int launch_scan(ScanP& p, int64_t heads, int64_t vdim, int64_t n_state, c
     } else {
         p.mode = 1;
         SCAN_ANY
-        if (p.vec) hipLaunchKernelGGL(k_seg_decay_prod, dim3((unsigned)(b->n_seq * n_seg), (unsigned)heads), dim3(256), 0, hs, p, *b);
+        if (p.vec) hipLaunchKernelGGL(k_seg_decay_prod, dim3((unsigned)(b->n_seq * n_seg), (unsigned)heads), dim3(1024), 0, hs, p, *b);
         const int64_t want_z = (1024 + b->n_seq * heads - 1) / (b->n_seq * heads), have_z = (n_state * vdim + 255) / 256;
         hipLaunchKernelGGL(k_ssm_seg_combine, dim3(b->n_seq, (unsigned)heads, (unsigned)(want_z < have_z ? want_z : have_z)), dim3(256), 0, hs, p, *b);
         p.mode = 2;
