@@ -607,9 +607,9 @@ GUTIVIK_BENCH_SIZES = {
     #       (plain + rotated) key size, latent rank; gated-linear-attention heads x key size x value size, rank of the decay's projection pair;
     #       experts x their ff, picks, groups.  Head counts, windows and experts are those of RETOTAR_BENCH_SIZES, so the stacks beside them
     #       move the same weights per token.
-    "1b": dict(width=2048, heads=16, kv_heads=4, dim=128, window=1024, keep=4, taps=4, rot=64, l_dim=128, l_rot=64, rank=512,
+    "1b": dict(width=2048, heads=16, kv_heads=4, dim=128, window=1024, keep=8, taps=4, rot=64, l_dim=128, l_rot=64, rank=512,
                g_heads=16, g_dim=128, g_vdim=128, low=16, experts=16, ff=1360, top=4, groups=4, keep_groups=2),
-    "8b": dict(width=4096, heads=32, kv_heads=8, dim=128, window=1024, keep=4, taps=4, rot=64, l_dim=128, l_rot=64, rank=512,
+    "8b": dict(width=4096, heads=32, kv_heads=8, dim=128, window=1024, keep=8, taps=4, rot=64, l_dim=128, l_rot=64, rank=512,
                g_heads=32, g_dim=128, g_vdim=128, low=16, experts=32, ff=2384, top=4, groups=4, keep_groups=2),
 }
 
@@ -661,15 +661,15 @@ def bench_gutivik(args, dev):
         mlp = dict(kind="moe", expert=dict(ff=z["ff"], limit=7.0), router=dict(experts=z["experts"], top=z["top"],
                                                                                groups=dict(count=z["groups"], keep=z["keep_groups"])))
         att = dict(heads=z["heads"], kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["dim"], scale=z["dim"] ** -0.5, conv=z["taps"],
-                   mask=dict(size=z["window"], keep_first=z["keep"]), rot=dict(dims=z["rot"], base=5e5), v_mix=True)
+                   mask=dict(size=z["window"], keep_first=z["keep"]), rot=dict(dims=z["rot"], base=1e6), v_mix=True)
         lat = dict(heads=z["heads"], dim=z["l_dim"], rot_dim=z["l_rot"], vdim=z["dim"], kv_rank=z["rank"], scale=(z["l_dim"] + z["l_rot"]) ** -0.5,
                    mask=dict(size=z["window"]), rot=dict(dims=z["l_rot"], base=1e4))
-        gla = dict(heads=z["g_heads"], dim=z["g_dim"], vdim=z["g_vdim"], tau=16.0)
+        gla = dict(heads=z["g_heads"], dim=z["g_dim"], vdim=z["g_vdim"], tau=8.0)
         A, L, G = (GutivikLayerConfig(t, m, mlp) for t, m in (("attention", att), ("latent_attention", lat), ("gla", gla)))
         for label, layers in (("attention x4", [A] * 4), ("latent_attention x4", [L] * 4), ("gla x4", [G] * 4), ("hybrid (a, l, g, a)", [A, L, G, A])):
             if args.only and args.only not in "gutivik " + label:
                 continue
-            model = GutivikModel(GutivikConfig(vocab, z["width"], 1e-6, 0.25, 30.0, 1 << 24, layers), "bfloat16", dev).init_random(1)
+            model = GutivikModel(GutivikConfig(vocab, z["width"], 1e-6, 0.5, 20.0, 1 << 24, layers), "bfloat16", dev).init_random(1)
             measure("gutivik " + label, name, model)
             del model
         r = RETOTAR_BENCH_SIZES[name]

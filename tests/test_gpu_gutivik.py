@@ -172,7 +172,7 @@ def test_rms_norm_alone_and_fused_with_the_residual_sum(dev):
 def test_scaled_and_capped_logits(dev):
     from zhilight_amd import seqops
     z = torch.linspace(-300, 300, 1001)
-    assert rel(seqops.scale_softcap(z.clone().to(dev), 0.25, 30.0), 30.0 * torch.tanh(z.double() * 0.25 / 30.0)) < 1e-6
+    assert rel(seqops.scale_softcap(z.clone().to(dev), 0.4, 25.0), 25.0 * torch.tanh(z.double() * 0.4 / 25.0)) < 1e-6
     assert rel(seqops.scale_softcap(z.clone().to(dev), 0.5, 0.0), z.double() * 0.5) < 1e-7
 
 
@@ -182,7 +182,7 @@ def test_gated_activations(dev):
     gu = (torch.randn(5, 2 * 48, generator=g) * 3).to(dev)
     a, u = gu.double().cpu()[:, :48], gu.double().cpu()[:, 48:]
     assert rel(seqops.act_mul(gu, torch.float32, kind="gelu_tanh"), O.gelu_tanh(a) * u) < 1e-6
-    lim = 1.5
+    lim = 1.3
     ref = torch.clamp(a, max=lim) * torch.sigmoid(1.702 * torch.clamp(a, max=lim)) * (torch.clamp(u, -lim, lim) + 1.0)
     assert rel(seqops.act_mul(gu, torch.float32, kind="swish_clamp", alpha=1.702, limit=lim), ref) < 1e-6
     assert rel(seqops.act_mul(gu, torch.float32, kind="silu"), a * torch.sigmoid(a) * u) < 1e-6
@@ -389,7 +389,7 @@ def test_latent_attention_with_a_wide_latent(dev, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads,dim,vdim,tau", [(2, 40, 24, 8.0), (1, 70, 9, 1.0), (3, 16, 64, 16.0), (2, 128, 128, 4.0)])
+@pytest.mark.parametrize("heads,dim,vdim,tau", [(2, 40, 24, 8.0), (1, 70, 9, 1.0), (3, 16, 64, 12.0), (2, 128, 128, 4.0)])
 def test_gated_linear_attention_in_portions_and_segments(dev, dtype, heads, dim, vdim, tau):
     layer = gla_cfg(heads, dim, vdim, tau)
     W, T = 80, 150
@@ -421,7 +421,7 @@ def test_decay_from_the_low_rank_pair_stays_in_fp32(dev):
         assert float(((got.cpu().double() - ref).abs() / ref).max()) < 1e-5
 
 
-@pytest.mark.parametrize("experts,count,keep,top", [(12, 3, 2, 2), (16, 2, 1, 3), (8, 4, 2, 3), (6, 6, 4, 3), (5, 1, 1, 1), (9, 3, 3, 4)])
+@pytest.mark.parametrize("experts,count,keep,top", [(12, 3, 2, 2), (16, 4, 1, 3), (8, 4, 2, 3), (6, 6, 4, 3), (5, 1, 1, 1), (9, 3, 3, 4)])
 def test_router_choice_against_the_restatement(dev, experts, count, keep, top):
     from zhilight_amd import seqops
     f = moe(experts=experts, count=count, keep=keep, top=top)
@@ -580,10 +580,10 @@ def test_router_choices_through_the_model_in_fp32(dev):
 
 def test_medium_configuration_other_kernel_instantiations(dev):
     """head sizes up to 128, a latent of 256 + 64, 16 heads on 4 kv heads, 32 experts in 8 groups, a portion long enough for scan segments"""
-    cfg = model_cfg([with_mlp(attention_cfg(heads=16, kv_heads=4, dim=128, vdim=64, conv=4, rot=64, size=200, keep=4, scale=0.09), dense(512)),
+    cfg = model_cfg([with_mlp(attention_cfg(heads=16, kv_heads=4, dim=128, vdim=64, conv=4, rot=64, size=200, keep=6, scale=0.09), dense(512)),
                      with_mlp(latent_cfg(heads=8, dim=64, rot=64, vdim=64, rank=256, size=100, scale=0.09), moe(ff=64, limit=2.0, experts=32, count=8, keep=3, top=4)),
-                     with_mlp(gla_cfg(heads=4, dim=64, vdim=128, tau=16.0), moe(ff=64, limit=2.0, experts=32, count=8, keep=3, top=4)),
-                     attention_cfg(heads=16, kv_heads=4, dim=128, vdim=64, conv=4, rot=64, size=200, keep=4, scale=0.09)],
+                     with_mlp(gla_cfg(heads=4, dim=64, vdim=128, tau=12.0), moe(ff=64, limit=2.0, experts=32, count=8, keep=3, top=4)),
+                     attention_cfg(heads=16, kv_heads=4, dim=128, vdim=64, conv=4, rot=64, size=200, keep=6, scale=0.09)],
                     width=256, vocab=300)
     sd = O.random_weights(cfg, 29, fixed_choice=True)
     toks = tokens_of(cfg, 420, 30)
