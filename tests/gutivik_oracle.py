@@ -228,8 +228,9 @@ def model(cfg, weights, tokens, round_to=None):
 
 def random_weights(cfg, seed=0, fixed_choice=False, low=8):
     """every tensor the configuration asks for, bf16-representable values (both serving formats start from the same numbers).
-    fixed_choice: the routers' correction terms lie more than 1 apart, so that they alone order the choice scores (sigmoid scores lie in
-    (0, 1)) and no choice is a close call under a rounded router input; the weights of the chosen experts still follow the scores."""
+    fixed_choice: the routers' correction terms are distinct powers of two times 1.25 -- more than 1 apart, and the sums of any two are
+    distinct as well -- so that they alone order the choice scores AND the groups' scores (sigmoid scores lie in (0, 1)): no choice is
+    a close call under a rounded router input; the weights of the chosen experts still follow the scores."""
     g = torch.Generator().manual_seed(seed)
     W = cfg["width"]
     sd = {}
@@ -284,7 +285,7 @@ def random_weights(cfg, seed=0, fixed_choice=False, low=8):
             E, ff = f["router"]["experts"], f["expert"]["ff"]
             mat(p + "mlp.router", E, W)
             if fixed_choice:
-                sd[p + "mlp.correction"] = (torch.randperm(E, generator=g).double() * 1.25).to(torch.bfloat16)
+                sd[p + "mlp.correction"] = (1.25 * 2.0 ** torch.randperm(E, generator=g).double()).to(torch.bfloat16)
             else:
                 vec(p + "mlp.correction", E, 0.3)
             for e in range(E):
