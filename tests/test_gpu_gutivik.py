@@ -285,6 +285,18 @@ def test_attention_one_far_key_across_pages_without_window(dev, dtype):
         assert_close(got.reshape(T, -1), ref.reshape(T, -1), dtype, j)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("d,e", [(8, 16), (72, 48), (160, 16), (256, 128)])
+def test_attention_head_sizes(dev, dtype, d, e):
+    """the other instantiations of the matrix-core kernel (32-coordinate steps of the head size) and long heads in the plain kernel"""
+    T, H, G = 200, 4, 2
+    q, k, v = aimed(T, H, G, d, e, [(150, 101), (199, 100), (120, 2), (190, 3)], d)
+    sink = torch.tensor([0.0, 1.0, -2.0, 0.5])
+    ref = O.softmax_attention(q, k, v, d ** -0.5, O.visible(T, 50, 3), sink.double())
+    got = attention_kernels(q, k, v, 50, 3, sink, d ** -0.5, dtype, dev, [130, 1, 1, 68])
+    assert_close(got.reshape(T, -1), ref.reshape(T, -1), dtype, (d, e))
+
+
 def build_mixer(layer, sd, prefix, width, dtype, dev, cache, source=None):
     from zhilight_amd import gutivik
     class L:                                                                    # what a builder looks at in the earlier layers
@@ -374,9 +386,12 @@ def test_latent_attention_rotated_part_and_window_edges(dev, dtype, window):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_latent_attention_with_a_wide_latent(dev, dtype):
-    """a cached row of 512 + 64 numbers (another instantiation of the single-token kernel), heads of 64 + 64"""
-    layer = latent_cfg(heads=3, dim=64, rot=64, vdim=48, rank=512, size=90, scale=0.09)
+@pytest.mark.parametrize("heads,dim,rot,vdim,rank", [(3, 64, 64, 48, 512), (2, 128, 64, 128, 64), (2, 200, 32, 72, 40), (1, 16, 8, 20, 24),
+                                                     (2, 24, 8, 40, 32), (2, 100, 20, 128, 48), (2, 200, 40, 200, 48)])
+def test_latent_attention_head_and_latent_sizes(dev, dtype, heads, dim, rot, vdim, rank):
+    """every instantiation of the prompt kernel (key and value sizes apart) and of the single-token kernels, up to a cached row of
+    512 + 64 numbers"""
+    layer = latent_cfg(heads=heads, dim=dim, rot=rot, vdim=vdim, rank=rank, size=90, scale=(dim + rot) ** -0.5)
     W, T = 128, 200
     cfg = model_cfg([layer], width=W)
     sd = O.random_weights(cfg, 9)
