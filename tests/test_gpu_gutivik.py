@@ -404,7 +404,7 @@ def test_latent_attention_head_and_latent_sizes(dev, dtype, heads, dim, rot, vdi
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads,dim,vdim,tau", [(2, 40, 24, 8.0), (1, 70, 9, 1.0), (3, 16, 64, 12.0), (2, 128, 128, 4.0)])
+@pytest.mark.parametrize("heads,dim,vdim,tau", [(2, 40, 24, 8.0), (1, 70, 9, 1.0), (3, 16, 64, 12.0), (2, 128, 128, 4.0), (2, 8, 16, 2.0), (1, 256, 96, 4.0)])
 def test_gated_linear_attention_in_portions_and_segments(dev, dtype, heads, dim, vdim, tau):
     layer = gla_cfg(heads, dim, vdim, tau)
     W, T = 80, 150
