@@ -77,10 +77,11 @@ int zls_latent_store(const float* proj, int64_t ld, int64_t col0, const float* w
 /* The same with a rotated key part: the down-projection holds rank + rot numbers from col0; the first rank are normed as above, the last
  * rot (one key part shared by all heads) are turned by the token's position -- pair (2i, 2i + 1) when interleaved, else (i, i + rot / 2),
  * by the angle p * freq[i] (freq fp32 (rot / 2)) -- and stored behind the latent: cache rows hold rank + rot numbers.  The last rot of the
- * qdim coordinates of each of the `heads` query heads (proj[t] from q_col0) are turned the same way in place. */
+ * qdim coordinates of each of the `heads` query heads (proj[t] from q_col0) are turned the same way in place.  cos and sin are multiplied
+ * by rot_gain (1: a plain rotation; frequencies rescaled for longer contexts come with a gain). */
 int zls_latent_rope_store(float* proj, int64_t ld, int64_t col0, const float* weight, float eps, int64_t rank, int64_t rot, const float* freq,
-                          int interleaved, int64_t q_col0, int64_t heads, int64_t qdim, const zls_batch_t* b, void* cache, int dtype,
-                          zl_stream_t s);
+                          int interleaved, int64_t q_col0, int64_t heads, int64_t qdim, float rot_gain, const zls_batch_t* b, void* cache,
+                          int dtype, zl_stream_t s);
 
 /* Causal attention of every token over its sequence's cached latents c_0 .. c_p, heads sharing the latent:
  *   score_j = scale * (W_uk,h^T q_h) . c_j;  w_j = exp(score_j) / (sum_i exp(score_i) + exp(sink_h));  o_h = W_uv,h (sum_j w_j c_j)
@@ -178,11 +179,27 @@ int zls_add_layer_norm(float* x, const float* y, const float* w, const float* b,
  * another layer's cache.  qk_freq fp32 (rot_dims / 2; rot_dims even, <= dim; 0: no rotation), v_freq fp32 (vdim / 2; vdim even).
  * dim, vdim <= 512.  interleaved != 0: the rotated pairs are the neighbours (2i, 2i + 1) instead of (i, i + rot_dims / 2), pair i turned by
  * p * qk_freq[i] either way.  vmix_src (nullable, fp32 rows of vmix_ld numbers): the values become (1 - vmix_lambda) v + vmix_lambda *
- * vmix_src[t][vmix_col0 ..] (kv_heads * vdim numbers of the same token, e.g. an earlier layer's values) before they are cached. */
+ * vmix_src[t][vmix_col0 ..] (kv_heads * vdim numbers of the same token, e.g. an earlier layer's values) before they are cached.
+ * q_norm_w / k_norm_w (nullable, fp32 (dim), shared by the heads; with qk_norm): the normed head is multiplied by the weight. */
 int zls_rope_norm_store(float* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, int64_t heads, int64_t kv_heads, int64_t dim,
                         int64_t vdim, const float* qk_freq, int64_t rot_dims, const float* v_freq, float eps, int qk_norm, int interleaved,
-                        const float* vmix_src, int64_t vmix_ld, int64_t vmix_col0, float vmix_lambda, const zls_batch_t* b, void* k_cache,
-                        void* v_cache, int dtype, zl_stream_t s);
+                        const float* vmix_src, int64_t vmix_ld, int64_t vmix_col0, float vmix_lambda, const float* q_norm_w, const float* k_norm_w,
+                        const zls_batch_t* b, void* k_cache, void* v_cache, int dtype, zl_stream_t s);
+
+/* The optional score form of the two attention launches below (NULL: plain scaled scores and a softmax).  For query head g at position p
+ * and key j:  s = scale * head_scale[g] * q.k;  s <- softcap * tanh(s / softcap) (softcap > 0);  s += bias[g][min(p - j, bias_rows - 1)];
+ * chunk > 0: only keys with j / chunk == p / chunk are visible (chunks counted from position 0; not together with keep_first);
+ * sigmoid != 0: the weight of a visible key is sigmoid(s + offset[g]), every key on its own -- nothing is normalised, a split leaves
+ * acc = sum_j w_j v_j and ml = (0, 1), and zls_head_mix_gate is called with plain_sum.  All pointers fp32 and nullable. */
+typedef struct {
+    const float* head_scale;   /* (heads) */
+    float softcap;
+    const float* bias;         /* (heads, bias_rows) */
+    int32_t bias_rows;
+    const float* offset;       /* (heads) */
+    int32_t chunk;
+    int32_t sigmoid;
+} zls_score_form_t;
 
 /* Softmax attention of every token over the cached keys j of its sequence with 0 <= p - j < window (window <= 0: all j <= p), and with
  * window > 0 also over the kept first keys j < keep_first (j <= p), at their true positions:
@@ -199,23 +216,25 @@ int zls_rope_norm_store(float* proj, int64_t ld, int64_t q_col0, int64_t k_col0,
  * and a multiple of 8. */
 int zls_window_attention(const float* q, int64_t ldq, int64_t q_col0, const void* k_cache, const void* v_cache, const zls_batch_t* b,
                          float scale, int64_t window, int64_t keep_first, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim, int all_kv,
-                         float* acc, float* ml, int64_t n_splits, int64_t pages_per_split, int single_only, int dtype, zl_stream_t s);
+                         float* acc, float* ml, int64_t n_splits, int64_t pages_per_split, int single_only, const zls_score_form_t* form,
+                         int dtype, zl_stream_t s);
 /* The same attention for query TILES on the matrix cores, bf16 only: tile i = tiles[3 i ..] = (first flat token, rows <= 64, sequence
  * index), consecutive tokens of one sequence.  Writes split 0 of acc for its tokens, unnormalised with ml = (m, sum) like the plain
  * kernel, and ml = (-inf, 0) for the other splits.  page_size 64, dim % 8 == 0, dim <= 256, vdim % 16 == 0. */
 int zls_window_attention_prompt(const float* q, int64_t ldq, int64_t q_col0, const void* k_cache, const void* v_cache, const zls_batch_t* b,
                                 const int32_t* tiles, int64_t n_tiles, float scale, int64_t window, int64_t keep_first, int64_t heads,
-                                int64_t kv_heads, int64_t dim, int64_t vdim, int all_kv, float* acc, float* ml, int64_t n_splits, int dtype,
-                                zl_stream_t s);
+                                int64_t kv_heads, int64_t dim, int64_t vdim, int all_kv, float* acc, float* ml, int64_t n_splits,
+                                const zls_score_form_t* form, int dtype, zl_stream_t s);
 
 /* out[t][h][:] = turn_back(sum_g talk[h][g] a[t][g][c(h)][:]) * sigmoid(gate[t][h * vdim + :]), a = the splits of acc merged:
  * a[t][g] = sum_s e^(m_s - M) acc[t][g][s] / (sum_s e^(m_s - M) l_s + e^(sink_g - M)), the last term only with sink (fp32 (heads),
  * nullable: a learned score per head that has no key and no value and is not scaled; M then also covers it).
  * talk fp32 (heads, heads), NULL: no mixing, acc holds vdim numbers per head and split; v_freq (nullable): pair (m, m + vdim / 2) is turned
- * by -p * v_freq[m]; gate fp32 (n_tok, ldg) from g_col0, NULL: no gate; out (n_tok, heads * vdim) in `dtype`. */
+ * by -p * v_freq[m]; gate fp32 (n_tok, ldg) from g_col0, NULL: no gate; out (n_tok, heads * vdim) in `dtype`.
+ * plain_sum != 0: the splits hold sums of finished weights (the sigmoid score form): a[t][g] = sum_s acc[t][g][s], no sink. */
 int zls_head_mix_gate(const float* acc, const float* ml, int64_t n_splits, const float* talk, const float* v_freq, const float* gate,
-                      int64_t ldg, int64_t g_col0, const float* sink, const zls_batch_t* b, int64_t heads, int64_t kv_heads, int64_t vdim, void* out,
-                      int dtype, zl_stream_t s);
+                      int64_t ldg, int64_t g_col0, const float* sink, int plain_sum, const zls_batch_t* b, int64_t heads, int64_t kv_heads,
+                      int64_t vdim, void* out, int dtype, zl_stream_t s);
 
 /* ---- linear attention with a scalar decay per head and token ---------------------------------------------------------------------- */
 /* S_t = a_t S_{t-1} + b_t k_t v_t^T,  y_t = S_t^T q_t   per head, S fp32 (dim x vdim) carried in state[slot].
@@ -257,9 +276,10 @@ int zls_lowrank_decay(const float* proj, int64_t ld, int64_t u_col0, int64_t low
  * correction (nullable); the outputs form `groups` equal groups of neighbours, a group's score is the sum of its `group_top` largest choice
  * scores (1: its largest), only outputs of the `keep` best groups can be chosen (groups <= 1: all) -- the others count as minus
  * infinity; the `top` largest choice scores are chosen (ties: the lower index).  ids int32 (n_tok, top), weights fp32 (n_tok, top) = s of
- * the chosen (divided by their sum + renorm_eps when renorm != 0).  n_out <= 1024, n_out % groups == 0. */
+ * the chosen (divided by their sum + renorm_eps when renorm != 0), times weight_scale.  n_out <= 1024, n_out % groups == 0. */
 int zls_moe_route(const float* logits, int64_t n_tok, int64_t n_out, const float* correction, int64_t groups, int64_t keep, int64_t top,
-                  int renorm, int score_kind, int64_t group_top, float renorm_eps, int32_t* ids, float* weights, zl_stream_t s);
+                  int renorm, int score_kind, int64_t group_top, float renorm_eps, float weight_scale, int32_t* ids, float* weights,
+                  zl_stream_t s);
 /* Sort the n_slots = n_tok * top (token, choice) pairs by expert: pairs whose id is >= n_experts (identity outputs) are left out.
  *   sorted_tok[p] = token of the pair at sorted position p;  slot_pos[t * top + k] = p (or -1);
  *   tiles[3 i ..] = (expert, first position, end position) of the i-th run of at most tile_m positions of one expert, expert = -1 for unused
@@ -287,6 +307,23 @@ int zls_act_mul(const float* gu, int64_t rows, int64_t ff, int kind, float alpha
  * h (n_tok, width) in `dtype`, out fp32. */
 int zls_moe_combine(const float* y, const int32_t* slot_pos, const int32_t* ids, const float* weights, const void* h, int64_t n_tok,
                     int64_t top, int64_t n_experts, int64_t width, float* out, int dtype, zl_stream_t s);
+
+/* ---- a residual kept as several streams ------------------------------------------------------------------------------------------ */
+/* The residual of a token is n <= 8 rows x_0 .. x_{n-1} of `width` fp32 numbers; element (t, s, i) of the streams that are READ lies at
+ * src[t * src_tok + s * src_stream + i] (src_stream = 0 reads one row as every stream: the start, where all streams equal the embedding).
+ * h[r] = N(sum_s read_coef[s] x_s[row r]) with N(u) = u / sqrt(mean(u^2) + eps) * (w + shift), row r = rows[r] (rows NULL: r);
+ * read_coef fp32 (n), NULL: all 1 (the sum of the streams); h (n_rows, width) in `dtype`.  The sum runs in the order of the streams. */
+int zls_streams_norm(const float* src, int64_t src_tok, int64_t src_stream, int64_t n, const float* read_coef, const int32_t* rows,
+                     const float* w, float shift, float eps, int64_t n_rows, int64_t width, void* h, int dtype, zl_stream_t s);
+/* A sub-layer's result y fp32 (n_tok, width) enters the streams:  y' = y * sigmoid(gate[t][g_col0 + i] + gate_bias[i]) (gate fp32 (n_tok,
+ * ldg), nullable: y' = y; gate_bias nullable);  x_d <- sum_s mix[s][d] x_s + out_coef[d] y' for every stream d at once from the old
+ * streams (mix fp32 (n, n) indexed [from][to], out_coef fp32 (n)); written to dst (n_tok, n, width), which may be src.  With read_coef
+ * (nullable) also h[t] = N(sum_d read_coef[d] x_d) of the NEW streams in `dtype`: the next sub-layer's input. */
+int zls_streams_update(const float* src, int64_t src_tok, int64_t src_stream, float* dst, int64_t n, const float* y, const float* gate,
+                       int64_t ldg, int64_t g_col0, const float* gate_bias, const float* mix, const float* out_coef, const float* read_coef,
+                       const float* w, float shift, float eps, int64_t n_tok, int64_t width, void* h, int dtype, zl_stream_t s);
+/* out[r][c] = act(z[r * ldz + c]) for fp32 z, out (rows, cols) in `dtype`: kind 0 relu(z)^2, 1 gelu_tanh(z), 2 silu(z). */
+int zls_unary_act(const float* z, int64_t ldz, int64_t rows, int64_t cols, int kind, void* out, int dtype, zl_stream_t s);
 
 #ifdef __cplusplus
 }

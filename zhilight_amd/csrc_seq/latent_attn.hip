@@ -23,7 +23,7 @@ namespace {
 template <int DT>
 __global__ __launch_bounds__(256) void k_latent_store(float* __restrict__ proj, int64_t ld, int col0, const float* __restrict__ weight,
                                                       float eps, int rank, int rot, const float* __restrict__ freq, int interleaved, int q_col0,
-                                                      int heads, int qdim, const zls_batch_t b, void* __restrict__ cache) {
+                                                      int heads, int qdim, const zls_batch_t b, void* __restrict__ cache, float rot_gain) {
     __shared__ float red[16];
     const int t = blockIdx.x;
     const int sq = b.tok_seq[t];
@@ -43,6 +43,7 @@ __global__ __launch_bounds__(256) void k_latent_store(float* __restrict__ proj, 
         const int a = interleaved ? 2 * i : i, c = interleaved ? 2 * i + 1 : i + half;
         float sn, cs;
         seq_sincos((float)pos * freq[i], &sn, &cs);
+        sn *= rot_gain; cs *= rot_gain;                                    // (rescaled frequencies come with a gain on cos and sin)
         float* src = vec == 0 ? row + col0 + rank : row + q_col0 + (size_t)(vec - 1) * qdim + (qdim - rot);
         const float x = src[a], y = src[c];
         const float xr = x * cs - y * sn, yr = y * cs + x * sn;
@@ -597,13 +598,13 @@ __global__ __launch_bounds__(64) void k_latent_decode_mfma(const AttnP p, const 
 }  // namespace
 
 extern "C" int zls_latent_rope_store(float* proj, int64_t ld, int64_t col0, const float* weight, float eps, int64_t rank, int64_t rot,
-                                     const float* freq, int interleaved, int64_t q_col0, int64_t heads, int64_t qdim, const zls_batch_t* b,
-                                     void* cache, int dtype, zl_stream_t s) {
+                                     const float* freq, int interleaved, int64_t q_col0, int64_t heads, int64_t qdim, float rot_gain,
+                                     const zls_batch_t* b, void* cache, int dtype, zl_stream_t s) {
     ZL_CHECK_ARG(proj && weight && cache && seq_batch_ok(b) && b->page_table && b->page_size > 0 && b->max_pages > 0 && rank > 0 && rot >= 0, ZL_EINVAL);
     ZL_CHECK_ARG(col0 >= 0 && col0 + rank + rot <= ld && rot % 2 == 0, ZL_ESHAPE);
     ZL_CHECK_ARG(rot == 0 || (freq && heads > 0 && qdim >= rot && q_col0 >= 0 && q_col0 + heads * qdim <= ld), ZL_ESHAPE);
 #define CALL(DT) hipLaunchKernelGGL((k_latent_store<DT>), dim3(b->n_tok), dim3(256), 0, (hipStream_t)s, proj, ld, (int)col0, weight, eps, (int)rank, \
-                                    (int)rot, freq, interleaved ? 1 : 0, (int)q_col0, (int)(rot ? heads : 0), (int)qdim, *b, cache);
+                                    (int)rot, freq, interleaved ? 1 : 0, (int)q_col0, (int)(rot ? heads : 0), (int)qdim, *b, cache, rot_gain);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
     return zl_launch_status();
@@ -611,7 +612,7 @@ extern "C" int zls_latent_rope_store(float* proj, int64_t ld, int64_t col0, cons
 
 extern "C" int zls_latent_store(const float* proj, int64_t ld, int64_t col0, const float* weight, float eps, int64_t rank, const zls_batch_t* b,
                                 void* cache, int dtype, zl_stream_t s) {
-    return zls_latent_rope_store(const_cast<float*>(proj), ld, col0, weight, eps, rank, 0, nullptr, 0, 0, 0, 0, b, cache, dtype, s);
+    return zls_latent_rope_store(const_cast<float*>(proj), ld, col0, weight, eps, rank, 0, nullptr, 0, 0, 0, 0, 1.0f, b, cache, dtype, s);
 }
 
 extern "C" int64_t zls_latent_attention_workspace_bytes(int64_t n_tok, int64_t heads, int64_t rank, int64_t n_splits) {

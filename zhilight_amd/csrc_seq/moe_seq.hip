@@ -3,7 +3,7 @@
 // k_moe_route    a wave per token: fp32 scores over all router outputs (softmax, or a sigmoid of each logit), choice scores = scores +
 //                correction, group-limited choice (a group's score = its best choice score, or the sum of its `group_top` best; outputs
 //                outside the best `keep` groups count as minus infinity), `top` picks by repeated arg-max (ties: the lower index),
-//                weights = the scores of the picks (optionally divided by their sum + renorm_eps)
+//                weights = the scores of the picks (optionally divided by their sum + renorm_eps), times weight_scale
 // k_moe_align    one workgroup: counts per expert, their prefix, every (token, choice) pair's place in the expert-sorted order, and the list of
 //                (expert, first, end) row tiles that the grouped product walks.  Identity outputs (id >= n_experts) take no place.
 // k_silu_mul     silu(gate) * up
@@ -24,7 +24,7 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {          // larg
 
 __global__ __launch_bounds__(64) void k_moe_route(const float* __restrict__ logits, int n_out, const float* __restrict__ correction, int groups,
                                                   int keep, int top, int renorm, int score_kind, int group_top, float renorm_eps,
-                                                  int32_t* __restrict__ ids, float* __restrict__ weights) {
+                                                  float weight_scale, int32_t* __restrict__ ids, float* __restrict__ weights) {
     __shared__ float prob[1024], choice[1024], gscore[1024];
     const int t = blockIdx.x, lane = threadIdx.x;
     const float* z = logits + (size_t)t * n_out;
@@ -100,9 +100,13 @@ __global__ __launch_bounds__(64) void k_moe_route(const float* __restrict__ logi
         wsum += prob[bi];
         __syncthreads();
     }
-    if (renorm) {
+    if (renorm || weight_scale != 1.0f) {
         __syncthreads();
-        for (int k = lane; k < top; k += 64) weights[(size_t)t * top + k] /= wsum + renorm_eps;
+        for (int k = lane; k < top; k += 64) {
+            float w = weights[(size_t)t * top + k];
+            if (renorm) w /= wsum + renorm_eps;
+            weights[(size_t)t * top + k] = w * weight_scale;
+        }
     }
 }
 
@@ -203,14 +207,15 @@ __global__ __launch_bounds__(256) void k_moe_combine(const float* __restrict__ y
 }  // namespace
 
 extern "C" int zls_moe_route(const float* logits, int64_t n_tok, int64_t n_out, const float* correction, int64_t groups, int64_t keep, int64_t top,
-                             int renorm, int score_kind, int64_t group_top, float renorm_eps, int32_t* ids, float* weights, zl_stream_t s) {
+                             int renorm, int score_kind, int64_t group_top, float renorm_eps, float weight_scale, int32_t* ids, float* weights,
+                             zl_stream_t s) {
     ZL_CHECK_ARG(logits && ids && weights && n_tok > 0 && n_out > 0 && top > 0, ZL_EINVAL);
     ZL_CHECK_ARG(n_out <= 1024 && top <= n_out, ZL_ELIMIT);
     if (groups < 1) groups = 1;
     ZL_CHECK_ARG(n_out % groups == 0 && keep >= 1 && keep <= groups && top <= keep * (n_out / groups), ZL_ESHAPE);
     ZL_CHECK_ARG((score_kind == 0 || score_kind == 1) && group_top >= 1, ZL_EINVAL);
     hipLaunchKernelGGL(k_moe_route, dim3((unsigned)n_tok), dim3(64), 0, (hipStream_t)s, logits, (int)n_out, correction, (int)groups, (int)keep,
-                       (int)top, renorm, score_kind, (int)group_top, renorm_eps, ids, weights);
+                       (int)top, renorm, score_kind, (int)group_top, renorm_eps, weight_scale, ids, weights);
     return zl_launch_status();
 }
 

@@ -1,6 +1,8 @@
 // seq_elem.hip -- the per-token steps between the matrix products of a ragged step: embedding with learned positions, token shift with
 // its carried row, the scalar-gain RMS norm fused with the residual sum, the gathered final norm, PolyNorm, layer norm, the weighted RMS
-// norm before a sub-layer (alone, or fused with the residual sum that precedes it), scaled and soft-capped logits.
+// norm before a sub-layer (alone, or fused with the residual sum that precedes it), scaled and soft-capped logits, and the same two steps
+// for a residual kept as SEVERAL streams (k_streams_norm, k_streams_update): a sub-layer reads a weighted sum of the streams, its result --
+// optionally gated by a sigmoid -- goes to every stream with a factor of its own while the streams are mixed by a small matrix.
 // One workgroup per token row; every sum of squares is fp32 (butterfly inside a wave, waves in order).
 #include "seq_common.h"
 
@@ -166,6 +168,87 @@ __global__ __launch_bounds__(kT) void k_scale_softcap(float* __restrict__ z, int
     z[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
 }
 
+constexpr int kMaxStreams = 8;
+
+struct StreamsP {
+    const float* src; int64_t src_tok, src_stream;      // the streams that are read: element (t, s, i) at t * src_tok + s * src_stream + i
+    float* dst;                                         // the streams that are written, (n_tok, n, width) -- may be src
+    int n, width;
+    const float* y;                                     // the sub-layer's result (n_tok, width)
+    const float* gate; int64_t ldg; int g_col0;         // nullable: y *= sigmoid(gate[t][g_col0 + i] + gate_bias[i])
+    const float* gate_bias;
+    const float* mix; const float* out_coef;            // (n, n) indexed [from][to]; (n)
+    const float* read_coef;                             // (n) nullable: the coefficients of the sum that is normed (NULL in k_streams_norm: all 1)
+    const int32_t* rows;                                // k_streams_norm: nullable gather
+    const float* w; float shift, eps;
+    void* h;                                            // the normed sum, (rows, width) in the serving format
+};
+
+// h[r] = norm(sum_s read_coef[s] x_s[row]) * (w + shift); the sum is taken in the order of the streams, fp32
+template <int DT>
+__global__ __launch_bounds__(kT) void k_streams_norm(const StreamsP p) {
+    extern __shared__ float u[];
+    __shared__ float red[16];
+    const size_t row = p.rows ? (size_t)p.rows[blockIdx.x] : (size_t)blockIdx.x;
+    const float* x = p.src + row * p.src_tok;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < p.width; i += kT) {
+        float a = 0.f;
+        for (int s = 0; s < p.n; ++s) a = fmaf(p.read_coef ? p.read_coef[s] : 1.0f, x[(size_t)s * p.src_stream + i], a);
+        u[i] = a;
+        ss = fmaf(a, a, ss);
+    }
+    const float f = 1.0f / sqrtf(zl_block_sum(ss, red) / (float)p.width + p.eps);
+    for (int i = threadIdx.x; i < p.width; i += kT) SeqT<DT>::st(p.h, (size_t)blockIdx.x * p.width + i, u[i] * f * (p.w[i] + p.shift));
+}
+
+// x_t <- sum_s mix[s][t] x_s + out_coef[t] * y * sigmoid(gate + bias), all streams from the old ones (a thread holds its element of every
+// stream in registers before it writes); with read_coef also the NEXT sub-layer's input, the normed weighted sum of the new streams
+template <int DT>
+__global__ __launch_bounds__(kT) void k_streams_update(const StreamsP p) {
+    extern __shared__ float u[];
+    __shared__ float red[16];
+    const size_t t = blockIdx.x;
+    const float* x = p.src + t * p.src_tok;
+    float* o = p.dst + t * (size_t)p.n * p.width;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < p.width; i += kT) {
+        float old[kMaxStreams];
+#pragma unroll
+        for (int s = 0; s < kMaxStreams; ++s) old[s] = s < p.n ? x[(size_t)s * p.src_stream + i] : 0.f;
+        float yv = p.y[t * p.width + i];
+        if (p.gate) yv *= seq_sigmoid(p.gate[t * p.ldg + p.g_col0 + i] + (p.gate_bias ? p.gate_bias[i] : 0.f));
+        float a = 0.f;
+        for (int d = 0; d < p.n; ++d) {
+            float v = 0.f;
+#pragma unroll
+            for (int s = 0; s < kMaxStreams; ++s)
+                if (s < p.n) v = fmaf(p.mix[s * p.n + d], old[s], v);
+            v = fmaf(p.out_coef[d], yv, v);
+            o[(size_t)d * p.width + i] = v;
+            if (p.read_coef) a = fmaf(p.read_coef[d], v, a);
+        }
+        u[i] = a;
+        ss = fmaf(a, a, ss);
+    }
+    if (!p.read_coef) return;
+    const float f = 1.0f / sqrtf(zl_block_sum(ss, red) / (float)p.width + p.eps);
+    for (int i = threadIdx.x; i < p.width; i += kT) SeqT<DT>::st(p.h, t * p.width + i, u[i] * f * (p.w[i] + p.shift));
+}
+
+// out = act(z): kind 0 relu(z)^2, 1 gelu_tanh(z), 2 silu(z)
+template <int DT>
+__global__ __launch_bounds__(kT) void k_unary_act(const float* __restrict__ z, int64_t ldz, int64_t rows, int64_t cols, int kind, void* __restrict__ out) {
+    const int64_t e = (int64_t)blockIdx.x * kT + threadIdx.x;
+    if (e >= rows * cols) return;
+    const float v = z[(e / cols) * ldz + e % cols];
+    float r;
+    if (kind == 0) { const float m = fmaxf(v, 0.f); r = m * m; }
+    else if (kind == 1) r = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    else r = seq_silu(v);
+    SeqT<DT>::st(out, (size_t)e, r);
+}
+
 }  // namespace
 
 extern "C" int zls_embed(const int32_t* tokens, const void* table, const void* pos_table, int64_t vocab, int64_t max_positions, float scale,
@@ -253,5 +336,45 @@ extern "C" int zls_add_rms_norm(float* x, const float* y, float eps, int64_t row
 extern "C" int zls_scale_softcap(float* z, int64_t n, float scale, float cap, zl_stream_t s) {
     ZL_CHECK_ARG(z && n > 0 && n < (1LL << 40), ZL_EINVAL);
     hipLaunchKernelGGL(k_scale_softcap, dim3((unsigned)((n + kT - 1) / kT)), dim3(kT), 0, (hipStream_t)s, z, n, scale, cap);
+    return zl_launch_status();
+}
+
+extern "C" int zls_streams_norm(const float* src, int64_t src_tok, int64_t src_stream, int64_t n, const float* read_coef, const int32_t* rows,
+                                const float* w, float shift, float eps, int64_t n_rows, int64_t width, void* h, int dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(src && w && h && n_rows > 0 && width > 0 && n > 0 && src_tok >= 0 && src_stream >= 0, ZL_EINVAL);
+    ZL_CHECK_ARG(n <= kMaxStreams && width * sizeof(float) <= 64 * 1024, ZL_ELIMIT);
+    StreamsP p = {};
+    p.src = src; p.src_tok = src_tok; p.src_stream = src_stream; p.n = (int)n; p.width = (int)width; p.read_coef = read_coef; p.rows = rows;
+    p.w = w; p.shift = shift; p.eps = eps; p.h = h;
+#define CALL(DT) hipLaunchKernelGGL((k_streams_norm<DT>), dim3((unsigned)n_rows), dim3(kT), (size_t)width * sizeof(float), (hipStream_t)s, p);
+    ZLS_DISPATCH(dtype, CALL)
+#undef CALL
+    return zl_launch_status();
+}
+
+extern "C" int zls_streams_update(const float* src, int64_t src_tok, int64_t src_stream, float* dst, int64_t n, const float* y, const float* gate,
+                                  int64_t ldg, int64_t g_col0, const float* gate_bias, const float* mix, const float* out_coef,
+                                  const float* read_coef, const float* w, float shift, float eps, int64_t n_tok, int64_t width, void* h, int dtype,
+                                  zl_stream_t s) {
+    ZL_CHECK_ARG(src && dst && y && mix && out_coef && n_tok > 0 && width > 0 && n > 0 && src_tok >= 0 && src_stream >= 0, ZL_EINVAL);
+    ZL_CHECK_ARG((!read_coef || (w && h)) && (!gate || (g_col0 >= 0 && g_col0 + width <= ldg)), ZL_ESHAPE);
+    ZL_CHECK_ARG(n <= kMaxStreams && width * sizeof(float) <= 64 * 1024, ZL_ELIMIT);
+    StreamsP p = {};
+    p.src = src; p.src_tok = src_tok; p.src_stream = src_stream; p.dst = dst; p.n = (int)n; p.width = (int)width; p.y = y; p.gate = gate;
+    p.ldg = ldg; p.g_col0 = (int)g_col0; p.gate_bias = gate_bias; p.mix = mix; p.out_coef = out_coef; p.read_coef = read_coef; p.w = w;
+    p.shift = shift; p.eps = eps; p.h = h;
+#define CALL(DT) hipLaunchKernelGGL((k_streams_update<DT>), dim3((unsigned)n_tok), dim3(kT), (size_t)width * sizeof(float), (hipStream_t)s, p);
+    ZLS_DISPATCH(dtype, CALL)
+#undef CALL
+    return zl_launch_status();
+}
+
+extern "C" int zls_unary_act(const float* z, int64_t ldz, int64_t rows, int64_t cols, int kind, void* out, int dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(z && out && rows > 0 && cols > 0 && ldz >= cols && kind >= 0 && kind <= 2, ZL_EINVAL);
+    const int64_t n = rows * cols;
+    ZL_CHECK_ARG(n < (1LL << 40), ZL_ELIMIT);
+#define CALL(DT) hipLaunchKernelGGL((k_unary_act<DT>), dim3((unsigned)((n + kT - 1) / kT)), dim3(kT), 0, (hipStream_t)s, z, ldz, rows, cols, kind, out);
+    ZLS_DISPATCH(dtype, CALL)
+#undef CALL
     return zl_launch_status();
 }

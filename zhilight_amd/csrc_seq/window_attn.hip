@@ -2,6 +2,9 @@
 // head (pairs half a part apart, or neighbouring coordinates), unit-RMS queries and keys, values turned by their own position and the sums
 // turned back, values blended with another layer's values of the same token, a sliding window that may keep the sequence's first keys, a
 // learned sink in the softmax denominator, weights mixed across heads after the softmax, a sigmoid gate per output coordinate.
+// A general score form (FORM = 1 instantiations) serves relatives: weighted query / key norms, a factor per head, scores capped by tanh, a
+// bias by the distance between query and key, queries confined to their chunk of positions, and weights that are sigmoids instead of a
+// softmax (every key on its own; the splits of a token are then plain sums).
 //
 // k_rope_norm_store    a workgroup per token, a wave per head in turn: the head's coordinates in registers, rotated, normed, written back
 //                      (queries, fp32, in place) or to the token's row of the paged planes (keys, values; serving format)
@@ -26,7 +29,7 @@ constexpr int kMaxV = 8;            // output coordinates per thread: (all_kv ? 
 // one head of `size` coordinates in the lanes' registers (coordinate i in lane i % 64, register i / 64): rotate the first n_rot (pairs
 // i, i + n_rot / 2; interleaved: pairs 2i, 2i + 1) by pos * freq[i], optionally divide by the root mean square; the result stays in v[]
 __device__ __forceinline__ void rope_head(float* v, const float* src, int size, int n_rot, const float* __restrict__ freq, float pos, bool norm,
-                                          float eps, int lane, bool interleaved = false) {
+                                          float eps, int lane, bool interleaved = false, const float* __restrict__ w = nullptr) {
     const int half = n_rot >> 1;
     float ss = 0.f;
 #pragma unroll
@@ -49,7 +52,7 @@ __device__ __forceinline__ void rope_head(float* v, const float* src, int size, 
     if (norm) {
         const float f = 1.0f / sqrtf(zl_wave_sum(ss) / (float)size + eps);
 #pragma unroll
-        for (int r = 0; r < kMaxE; ++r) v[r] *= f;
+        for (int r = 0; r < kMaxE; ++r) v[r] *= (w && lane + 64 * r < size) ? f * w[lane + 64 * r] : f;
     }
 }
 
@@ -61,6 +64,7 @@ struct RopeP {
     void* k_cache; void* v_cache;
     int interleaved;
     const float* vmix_src; int64_t vmix_ld; int vmix_col0; float vmix_lambda;     // values <- (1 - lambda) values + lambda vmix_src[t][col0 ..]
+    const float* q_w; const float* k_w;             // nullable (dim): weights of the query / key norm, shared by the heads
 };
 
 template <int DT>
@@ -77,13 +81,13 @@ __global__ __launch_bounds__(256) void k_rope_norm_store(const RopeP p, const zl
     for (int h = wave; h < p.heads + 2 * n_kv; h += 4) {                 // (a wave owns its heads: no two waves touch the same numbers)
         if (h < p.heads) {
             float* q = row + p.q_col0 + h * p.dim;
-            rope_head(v, q, p.dim, p.rot_dims, p.qk_freq, pos, p.qk_norm != 0, p.eps, lane, p.interleaved != 0);
+            rope_head(v, q, p.dim, p.rot_dims, p.qk_freq, pos, p.qk_norm != 0, p.eps, lane, p.interleaved != 0, p.q_w);
 #pragma unroll
             for (int r = 0; r < kMaxE; ++r)
                 if (lane + 64 * r < p.dim) q[lane + 64 * r] = v[r];
         } else if (h < p.heads + n_kv) {
             const int c = h - p.heads;
-            rope_head(v, row + p.k_col0 + c * p.dim, p.dim, p.rot_dims, p.qk_freq, pos, p.qk_norm != 0, p.eps, lane, p.interleaved != 0);
+            rope_head(v, row + p.k_col0 + c * p.dim, p.dim, p.rot_dims, p.qk_freq, pos, p.qk_norm != 0, p.eps, lane, p.interleaved != 0, p.k_w);
 #pragma unroll
             for (int r = 0; r < kMaxE; ++r)
                 if (lane + 64 * r < p.dim) SeqT<DT>::st(p.k_cache, (crow * p.kv_heads + c) * p.dim + lane + 64 * r, v[r]);
@@ -132,14 +136,28 @@ struct AttnP {
     float* acc; float* ml;                 // (n_tok, heads, n_splits, nv) partial sums | (n_tok, heads, n_splits, 2) their maximum and weight sum
     int n_splits, pages_per_split, single_only;
     const int32_t* tiles;                  // the matrix-core kernel: (first flat token, rows, sequence) per query tile
+    // the general score form (kernels instantiated with FORM = 1; all of it optional):
+    const float* head_scale;               // (heads) the score of head g is also multiplied by head_scale[g]
+    float softcap;                         // > 0: score <- softcap * tanh(score / softcap)
+    const float* bias; int bias_rows;      // (heads, bias_rows): bias[g][min(p - j, bias_rows - 1)] is added to the (capped) score
+    const float* offset;                   // (heads) sigmoid weights: w = sigmoid(score + offset[g])
+    int chunk;                             // > 0: a query only sees the keys of its own chunk of `chunk` positions, counted from position 0
+    int sigmoid;                           // weights are sigmoids, each key on its own: no maximum, no normaliser (ml = (0, 1) for a split with keys)
 };
+
+// the score of the general form from the scaled product
+__device__ __forceinline__ float form_score(const AttnP& p, float s, int g, int dist) {
+    if (p.softcap > 0.f) s = p.softcap * tanhf(s / p.softcap);
+    if (p.bias) s += p.bias[(size_t)g * p.bias_rows + min(dist, p.bias_rows - 1)];
+    return s;
+}
 
 // A token's pages: those that only hold kept first keys (before the page of the window's oldest key), then the window's.  Split s walks
 // pages_per_split of that list from s * pages_per_split, a page at a
 // time: scores of the page's keys (a wave per key), weights with the running maximum -- 0 for keys outside the window or after the
 // token -- then every thread adds the WHOLE page of its value coordinates (the plane holds values transposed, 8 keys per 16-byte load).
 // What a split leaves is unnormalised: sum_j e^(s_j - m) v_j with m and sum_j e^(s_j - m); k_head_mix_gate merges the splits.
-template <int DT>
+template <int DT, int FORM>
 __global__ __launch_bounds__(256) void k_window_attention(const AttnP p, const zls_batch_t b) {
     extern __shared__ float lds[];
     __shared__ float red[16];
@@ -150,13 +168,15 @@ __global__ __launch_bounds__(256) void k_window_attention(const AttnP p, const z
     if (p.single_only && b.seq_start[sq + 1] - b.seq_start[sq] > 1) return;
     const int ps = b.page_size;
     const int pos = b.seq_pos0[sq] + (t - b.seq_start[sq]);
-    const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+    int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+    if (FORM && p.chunk > 0) lo = max(lo, pos / p.chunk * p.chunk);
     const int wp0 = lo / ps, nkp = min((p.keep_first + ps - 1) / ps, wp0);   // kept pages before the window's first page
     const int c = g / (p.heads / p.kv_heads);
     const int nv = p.all_kv ? p.kv_heads * p.vdim : p.vdim, voff = p.all_kv ? 0 : c * p.vdim;
     const int32_t* pages = b.page_table + (size_t)sq * b.max_pages;
     const int li0 = sp * p.pages_per_split, li1 = min(nkp + pos / ps - wp0, li0 + p.pages_per_split - 1);
-    for (int i = tid; i < p.dim; i += 256) qs[i] = p.q[(size_t)t * p.ldq + p.q_col0 + g * p.dim + i] * p.scale;
+    const float qscale = (FORM && p.head_scale) ? p.scale * p.head_scale[g] : p.scale;
+    for (int i = tid; i < p.dim; i += 256) qs[i] = p.q[(size_t)t * p.ldq + p.q_col0 + g * p.dim + i] * qscale;
     float A[kMaxV];
 #pragma unroll
     for (int r = 0; r < kMaxV; ++r) A[r] = 0.f;
@@ -174,10 +194,35 @@ __global__ __launch_bounds__(256) void k_window_attention(const AttnP p, const z
                 part = 0.f;
                 for (int i = lane; i < p.dim; i += 64) part = fmaf(qs[i], SeqT<DT>::ld(p.k_cache, at + i), part);
                 part = zl_wave_sum(part);
+                if (FORM) part = form_score(p, part, g, pos - j);
             }
             if (lane == 0) sc[jj] = part;
         }
         __syncthreads();
+        if (FORM && p.sigmoid) {                                          // every key on its own: no maximum, nothing to correct
+            const float off = p.offset ? p.offset[g] : 0.f;
+            for (int jj = tid; jj < ps; jj += 256) sc[jj] = sc[jj] == -INFINITY ? 0.f : seq_sigmoid(sc[jj] + off);
+            m = 0.f; l = 1.f;
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < kMaxV; ++r) {
+                const int e = tid + 256 * r;
+                if (e < nv) {
+                    float a = A[r];
+                    const size_t at = (page * p.kv_heads * p.vdim + voff + e) * ps;
+                    for (int j8 = 0; j8 < ps; j8 += 8) {
+                        float v[8];
+                        Ld8<DT>::ld(p.v_cache, at + j8, v);
+                        const float4 w0 = *reinterpret_cast<const float4*>(sc + j8), w1 = *reinterpret_cast<const float4*>(sc + j8 + 4);
+                        a = fmaf(w0.x, v[0], a); a = fmaf(w0.y, v[1], a); a = fmaf(w0.z, v[2], a); a = fmaf(w0.w, v[3], a);
+                        a = fmaf(w1.x, v[4], a); a = fmaf(w1.y, v[5], a); a = fmaf(w1.z, v[6], a); a = fmaf(w1.w, v[7], a);
+                    }
+                    A[r] = a;
+                }
+            }
+            __syncthreads();
+            continue;
+        }
         float cm = -INFINITY;
         for (int jj = tid; jj < ps; jj += 256) cm = fmaxf(cm, sc[jj]);
         const float m_new = fmaxf(m, zl_block_max(cm, red));              // finite: the page holds a visible key
@@ -245,10 +290,19 @@ __device__ __forceinline__ void split8(const float* v, uint4& hi, uint4& lo) {
     lo = make_uint4(l[0] | l[1] << 16, l[2] | l[3] << 16, l[4] | l[5] << 16, l[6] | l[7] << 16);
 }
 
-template <int KS>                       // 32-coordinate steps of the head size: dim <= 32 KS
+constexpr int kBiasLds = 2048;          // rows of a head's distance bias that the matrix-core kernel keeps in LDS (longer tables: the rest from memory)
+
+// tanh and the logistic function on the hardware's exp2 and reciprocal: 1 ulp each, far inside what bf16 keys leave (bf16 kernel only)
+__device__ __forceinline__ float fast_sigmoid(float x) {
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+}
+__device__ __forceinline__ float fast_tanh(float x) { return 2.0f * fast_sigmoid(2.0f * x) - 1.0f; }
+
+template <int KS, int FORM>             // 32-coordinate steps of the head size: dim <= 32 KS; FORM 1: the general score form of AttnP
 __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, const zls_batch_t b) {
     __shared__ uint4 pfrag[2][4][2][2][64];                              // [buffer][query block][key half][hi, lo][lane]
     __shared__ float corr_s[2][64], l_s[64], m_s[64];
+    __shared__ float bias_s[FORM ? kBiasLds : 1];
     const int tile = blockIdx.x, g = blockIdx.y, part = blockIdx.z;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nrow = lane & 15, kq = lane >> 4;
     const int t0 = p.tiles[3 * tile], rows = p.tiles[3 * tile + 1], sq = p.tiles[3 * tile + 2];
@@ -263,6 +317,13 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
     const int qi = 16 * wave + nrow;
     const bool qok = qi < rows;
     const int pq = pos0 + qi;
+    const float qscale = (FORM && p.head_scale) ? p.scale * p.head_scale[g] : p.scale;
+    const int chunk0 = (FORM && p.chunk > 0) ? pq / p.chunk * p.chunk : 0;          // the first position of the query's chunk
+    const float off = (FORM && p.offset) ? p.offset[g] : 0.f;
+    if (FORM && p.bias) {
+        for (int i = tid; i < min(p.bias_rows, kBiasLds); i += 256) bias_s[i] = p.bias[(size_t)g * p.bias_rows + i];
+        __syncthreads();
+    }
     uint4 qh[KS], ql[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -270,7 +331,7 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int x = 32 * ks + 8 * kq + i;
-            v[i] = (qok && x < d) ? p.q[(size_t)(t0 + qi) * p.ldq + p.q_col0 + g * d + x] * p.scale : 0.f;
+            v[i] = (qok && x < d) ? p.q[(size_t)(t0 + qi) * p.ldq + p.q_col0 + g * d + x] * qscale : 0.f;
         }
         split8(v, qh[ks], ql[ks]);
     }
@@ -282,7 +343,9 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
 #pragma unroll
         for (int qb = 0; qb < 4; ++qb) acc[i][qb] = (f4v){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
-    const int lo_key = p.window > 0 ? max(0, pos0 - p.window + 1) : 0, hi_key = pos0 + rows - 1;
+    int lo_key = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
+    if (FORM && p.chunk > 0) lo_key = max(lo_key, pos0 / p.chunk * p.chunk);        // (the tile's first query has the oldest chunk)
+    const int hi_key = pos0 + rows - 1;
     int buf = 0;
     const int pg_last = hi_key / 64;
     // the key fragments of a page: A operands straight from the cache rows; the NEXT page's are requested as soon as this page's scores
@@ -325,26 +388,36 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int j = pg * 64 + 16 * kb + 4 * kq + r;
-                vis[kb][r] = qok && j <= pq && (p.window <= 0 || pq - j < p.window || j < p.keep_first);
+                vis[kb][r] = qok && j <= pq && (p.window <= 0 || pq - j < p.window || j < p.keep_first) && (!FORM || j >= chunk0);
+                if (FORM && vis[kb][r]) {
+                    float sv = st[kb][r];
+                    if (p.softcap > 0.f) sv = p.softcap * fast_tanh(sv * __builtin_amdgcn_rcpf(p.softcap));
+                    if (p.bias) {
+                        const int bi = min(pq - j, p.bias_rows - 1);
+                        sv += bi < kBiasLds ? bias_s[bi] : p.bias[(size_t)g * p.bias_rows + bi];
+                    }
+                    st[kb][r] = sv;
+                }
                 if (vis[kb][r]) cm = fmaxf(cm, st[kb][r]);
             }
         cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
         cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
-        const float m_new = fmaxf(m_run, cm);
+        const bool sig = FORM && p.sigmoid;
+        const float m_new = sig ? 0.f : fmaxf(m_run, cm);
         // (this kernel serves bf16 only: the hardware's exp2 is accurate to 1 ulp of the fp32 result, far inside what the bf16 keys leave)
         constexpr float kLog2e = 1.4426950408889634f;
-        const float corr = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f((m_run - m_new) * kLog2e);
+        const float corr = (sig || m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f((m_run - m_new) * kLog2e);
         float pw[4][4], psum = 0.f;
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                pw[kb][r] = vis[kb][r] ? __builtin_amdgcn_exp2f((st[kb][r] - m_new) * kLog2e) : 0.f;
+                pw[kb][r] = !vis[kb][r] ? 0.f : sig ? fast_sigmoid(st[kb][r] + off) : __builtin_amdgcn_exp2f((st[kb][r] - m_new) * kLog2e);
                 psum += pw[kb][r];
             }
         psum += __shfl_xor(psum, 16, 64);
         psum += __shfl_xor(psum, 32, 64);
-        l_run = l_run * corr + psum;
+        l_run = sig ? 1.0f : l_run * corr + psum;                         // (sigmoid weights: nothing to normalise, ml = (0, 1))
         m_run = m_new;
 #pragma unroll
         for (int h2 = 0; h2 < 2; ++h2) {
@@ -421,6 +494,7 @@ struct MixP {
     int heads, kv_heads, vdim, n_splits;
     void* out;
     const float* sink;                                                    // (heads) nullable: exp(sink_h) joins head h's denominator
+    int plain_sum;                                                        // the splits hold finished weights (sigmoids): they are added, not normalised
 };
 
 // a workgroup per (token, key / value head c): the splits of every source head merged into LDS (for c's values only), then for the heads of
@@ -443,6 +517,10 @@ __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_b
     if (S > 1)
         for (int k = threadIdx.x >> 6; k < n_src; k += 4) {               // a wave per source head, a lane per split: all loads at once
             const float2* mlp = reinterpret_cast<const float2*>(p.ml) + ((size_t)t * p.heads + src0 + k) * S;
+            if (p.plain_sum) {
+                for (int s = lane; s < S; s += 64) wsp[k * S + s] = mlp[s].y > 0.f ? 1.0f : 0.f;
+                continue;
+            }
             float M = p.sink ? p.sink[src0 + k] : -INFINITY;
             for (int s = lane; s < S; s += 64) M = fmaxf(M, mlp[s].x);
             M = zl_wave_max(M);
@@ -470,8 +548,8 @@ __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_b
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
                 const float* mlp = p.ml + 2 * ((size_t)t * p.heads + src0 + kk[r]);
-                float f = 1.0f / mlp[1];
-                if (p.sink) {
+                float f = p.plain_sum ? 1.0f : 1.0f / mlp[1];
+                if (p.sink && !p.plain_sum) {
                     const float sk = p.sink[src0 + kk[r]], M = fmaxf(mlp[0], sk), e = expf(mlp[0] - M);
                     f = e / (mlp[1] * e + expf(sk - M));
                 }
@@ -534,7 +612,8 @@ __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_b
 extern "C" int zls_rope_norm_store(float* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, int64_t heads, int64_t kv_heads,
                                    int64_t dim, int64_t vdim, const float* qk_freq, int64_t rot_dims, const float* v_freq, float eps, int qk_norm,
                                    int interleaved, const float* vmix_src, int64_t vmix_ld, int64_t vmix_col0, float vmix_lambda,
-                                   const zls_batch_t* b, void* k_cache, void* v_cache, int dtype, zl_stream_t s) {
+                                   const float* q_norm_w, const float* k_norm_w, const zls_batch_t* b, void* k_cache, void* v_cache, int dtype,
+                                   zl_stream_t s) {
     ZL_CHECK_ARG(proj && seq_batch_ok(b) && b->page_table && b->page_size > 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0, ZL_EINVAL);
     ZL_CHECK_ARG((k_cache == nullptr) == (v_cache == nullptr), ZL_EINVAL);
     ZL_CHECK_ARG(rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0 && (rot_dims == 0 || qk_freq) && (!v_freq || vdim % 2 == 0), ZL_ESHAPE);
@@ -546,6 +625,7 @@ extern "C" int zls_rope_norm_store(float* proj, int64_t ld, int64_t q_col0, int6
     p.kv_heads = (int)kv_heads; p.dim = (int)dim; p.vdim = (int)vdim; p.rot_dims = (int)rot_dims; p.qk_norm = qk_norm; p.qk_freq = qk_freq;
     p.v_freq = v_freq; p.eps = eps; p.k_cache = k_cache; p.v_cache = v_cache;
     ZL_CHECK_ARG(!vmix_src || (vmix_col0 >= 0 && vmix_col0 + kv_heads * vdim <= vmix_ld), ZL_ESHAPE);
+    p.q_w = qk_norm ? q_norm_w : nullptr; p.k_w = qk_norm ? k_norm_w : nullptr;
     p.interleaved = interleaved ? 1 : 0; p.vmix_src = vmix_src; p.vmix_ld = vmix_ld; p.vmix_col0 = (int)vmix_col0; p.vmix_lambda = vmix_lambda;
 #define CALL(DT) hipLaunchKernelGGL((k_rope_norm_store<DT>), dim3(b->n_tok), dim3(256), 0, (hipStream_t)s, p, *b);
     ZLS_DISPATCH(dtype, CALL)
@@ -553,10 +633,20 @@ extern "C" int zls_rope_norm_store(float* proj, int64_t ld, int64_t q_col0, int6
     return zl_launch_status();
 }
 
+// the optional score form of a launch (NULL: plain scaled scores and a softmax)
+static int set_form(AttnP& p, const zls_score_form_t* f) {
+    if (!f) return ZL_OK;
+    ZL_CHECK_ARG((!f->bias || f->bias_rows > 0) && f->chunk >= 0 && f->chunk < (1 << 30), ZL_ESHAPE);
+    ZL_CHECK_ARG(!(f->chunk > 0 && p.keep_first > 0), ZL_ESHAPE);        // (kept first keys belong to a sliding window, not to chunks)
+    p.head_scale = f->head_scale; p.softcap = f->softcap; p.bias = f->bias; p.bias_rows = f->bias_rows; p.offset = f->offset;
+    p.chunk = f->chunk; p.sigmoid = f->sigmoid ? 1 : 0;
+    return ZL_OK;
+}
+
 extern "C" int zls_window_attention(const float* q, int64_t ldq, int64_t q_col0, const void* k_cache, const void* v_cache, const zls_batch_t* b,
                                     float scale, int64_t window, int64_t keep_first, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
-                                    int all_kv, float* acc, float* ml, int64_t n_splits, int64_t pages_per_split, int single_only, int dtype,
-                                    zl_stream_t s) {
+                                    int all_kv, float* acc, float* ml, int64_t n_splits, int64_t pages_per_split, int single_only,
+                                    const zls_score_form_t* form, int dtype, zl_stream_t s) {
     ZL_CHECK_ARG(q && k_cache && v_cache && acc && ml && seq_batch_ok(b) && b->page_table && b->page_size > 0, ZL_EINVAL);
     ZL_CHECK_ARG(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0 && heads <= 65535, ZL_ESHAPE);
     ZL_CHECK_ARG(q_col0 >= 0 && q_col0 + heads * dim <= ldq && window < (1 << 30) && n_splits >= 1 && n_splits <= 65535 && pages_per_split >= 1 &&
@@ -567,8 +657,13 @@ extern "C" int zls_window_attention(const float* q, int64_t ldq, int64_t q_col0,
     p.heads = (int)heads; p.kv_heads = (int)kv_heads; p.dim = (int)dim; p.vdim = (int)vdim; p.all_kv = all_kv ? 1 : 0; p.acc = acc; p.ml = ml;
     p.n_splits = (int)n_splits; p.pages_per_split = (int)pages_per_split; p.single_only = single_only ? 1 : 0;
     p.keep_first = p.window > 0 ? (int)keep_first : 0;
+    const int st = set_form(p, form);
+    if (st != ZL_OK) return st;
     const size_t lds = (size_t)dim * sizeof(float);
-#define CALL(DT) hipLaunchKernelGGL((k_window_attention<DT>), dim3(b->n_tok, (unsigned)heads, (unsigned)n_splits), dim3(256), lds, (hipStream_t)s, p, *b);
+    const dim3 grid(b->n_tok, (unsigned)heads, (unsigned)n_splits);
+#define CALL(DT)                                                                                            \
+    if (form) hipLaunchKernelGGL((k_window_attention<DT, 1>), grid, dim3(256), lds, (hipStream_t)s, p, *b); \
+    else hipLaunchKernelGGL((k_window_attention<DT, 0>), grid, dim3(256), lds, (hipStream_t)s, p, *b);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
     return zl_launch_status();
@@ -577,7 +672,7 @@ extern "C" int zls_window_attention(const float* q, int64_t ldq, int64_t q_col0,
 extern "C" int zls_window_attention_prompt(const float* q, int64_t ldq, int64_t q_col0, const void* k_cache, const void* v_cache,
                                            const zls_batch_t* b, const int32_t* tiles, int64_t n_tiles, float scale, int64_t window,
                                            int64_t keep_first, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim, int all_kv, float* acc, float* ml, int64_t n_splits,
-                                           int dtype, zl_stream_t s) {
+                                           const zls_score_form_t* form, int dtype, zl_stream_t s) {
     ZL_CHECK_ARG(q && k_cache && v_cache && acc && ml && tiles && n_tiles > 0 && seq_batch_ok(b) && b->page_table, ZL_EINVAL);
     ZL_CHECK_ARG(dtype == ZL_BF16, ZL_EDTYPE);
     ZL_CHECK_ARG(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && heads <= 65535 && n_splits >= 1 && q_col0 >= 0 && q_col0 + heads * dim <= ldq,
@@ -588,23 +683,29 @@ extern "C" int zls_window_attention_prompt(const float* q, int64_t ldq, int64_t 
     p.q = q; p.ldq = ldq; p.q_col0 = (int)q_col0; p.k_cache = k_cache; p.v_cache = v_cache; p.scale = scale; p.window = (int)window;
     p.heads = (int)heads; p.kv_heads = (int)kv_heads; p.dim = (int)dim; p.vdim = (int)vdim; p.all_kv = all_kv ? 1 : 0; p.acc = acc; p.ml = ml;
     p.n_splits = (int)n_splits; p.tiles = tiles; p.keep_first = p.window > 0 ? (int)keep_first : 0;
+    const int st = set_form(p, form);
+    if (st != ZL_OK) return st;
     const int64_t n_blocks = (all_kv ? kv_heads : 1) * vdim / 16, parts = (n_blocks + 4 * kItems - 1) / (4 * kItems);
     ZL_CHECK_ARG(parts <= 65535, ZL_ELIMIT);
     const dim3 grid((unsigned)n_tiles, (unsigned)heads, (unsigned)parts);
     hipStream_t hs = (hipStream_t)s;
     const int ks = (int)((dim + 31) / 32);
-    if (ks <= 1) hipLaunchKernelGGL((k_window_attention_mfma<1>), grid, dim3(256), 0, hs, p, *b);
-    else if (ks <= 2) hipLaunchKernelGGL((k_window_attention_mfma<2>), grid, dim3(256), 0, hs, p, *b);
-    else if (ks <= 3) hipLaunchKernelGGL((k_window_attention_mfma<3>), grid, dim3(256), 0, hs, p, *b);
-    else if (ks <= 4) hipLaunchKernelGGL((k_window_attention_mfma<4>), grid, dim3(256), 0, hs, p, *b);
-    else if (ks <= 6) hipLaunchKernelGGL((k_window_attention_mfma<6>), grid, dim3(256), 0, hs, p, *b);
-    else hipLaunchKernelGGL((k_window_attention_mfma<8>), grid, dim3(256), 0, hs, p, *b);
+#define PROMPT(KS)                                                                                      \
+    if (form) hipLaunchKernelGGL((k_window_attention_mfma<KS, 1>), grid, dim3(256), 0, hs, p, *b);      \
+    else hipLaunchKernelGGL((k_window_attention_mfma<KS, 0>), grid, dim3(256), 0, hs, p, *b)
+    if (ks <= 1) { PROMPT(1); }
+    else if (ks <= 2) { PROMPT(2); }
+    else if (ks <= 3) { PROMPT(3); }
+    else if (ks <= 4) { PROMPT(4); }
+    else if (ks <= 6) { PROMPT(6); }
+    else { PROMPT(8); }
+#undef PROMPT
     return zl_launch_status();
 }
 
 extern "C" int zls_head_mix_gate(const float* acc, const float* ml, int64_t n_splits, const float* talk, const float* v_freq, const float* gate,
-                                 int64_t ldg, int64_t g_col0, const float* sink, const zls_batch_t* b, int64_t heads, int64_t kv_heads, int64_t vdim,
-                                 void* out, int dtype, zl_stream_t s) {
+                                 int64_t ldg, int64_t g_col0, const float* sink, int plain_sum, const zls_batch_t* b, int64_t heads,
+                                 int64_t kv_heads, int64_t vdim, void* out, int dtype, zl_stream_t s) {
     ZL_CHECK_ARG(acc && ml && out && seq_batch_ok(b) && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && vdim > 0 && n_splits >= 1, ZL_EINVAL);
     ZL_CHECK_ARG((!v_freq || vdim % 2 == 0) && (!gate || (g_col0 >= 0 && g_col0 + heads * vdim <= ldg)), ZL_ESHAPE);
     const int64_t n_src = talk ? heads : heads / kv_heads;
@@ -613,6 +714,7 @@ extern "C" int zls_head_mix_gate(const float* acc, const float* ml, int64_t n_sp
     MixP p;
     p.acc = acc; p.ml = ml; p.n_splits = (int)n_splits; p.talk = talk; p.v_freq = v_freq; p.gate = gate; p.ldg = ldg; p.g_col0 = (int)g_col0;
     p.heads = (int)heads; p.kv_heads = (int)kv_heads; p.vdim = (int)vdim; p.out = out; p.sink = sink;
+    p.plain_sum = plain_sum ? 1 : 0;
 #define CALL(DT) hipLaunchKernelGGL((k_head_mix_gate<DT>), dim3(b->n_tok, (unsigned)kv_heads), dim3(256), lds, (hipStream_t)s, p, *b);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL

@@ -32,20 +32,39 @@ def _rand(gen, shape, std, dtype, device):
     return (torch.randn(shape, generator=gen, device=device, dtype=torch.float32) * std).to(dtype)
 
 
-class LatentAttention:
+class SideRows:
+    """Mixers and feed-forwards whose first step is ONE product over their input can carry more rows in it for their caller: a layer that
+    needs another projection of the same input (a gate of the sub-layer's result, say) attaches its matrix after load / init_random and
+    finds the fp32 outputs in `side` = (tensor, first column) after forward -- one launch and one pass over the input less."""
+    side = None
+    side_col0 = None
+    _side_matrix = "w_in"
+
+    def attach_side(self, w):
+        m = getattr(self, self._side_matrix)
+        if w.shape[1] != m.shape[1] or w.dtype != m.dtype:
+            raise ZLError("side rows must have the input projection's width and format")
+        self.side_col0 = m.shape[0]
+        setattr(self, self._side_matrix, torch.cat([m, w], dim=0).contiguous())
+
+
+class LatentAttention(SideRows):
     """Causal attention whose keys and values are up-projections of a cached, RMS-normed low-rank latent; optional learned per-head sink in
     the softmax denominator, per-head sigmoid output gate, sliding window (`window` > 0: position p sees p - window < j <= p), and a
     ROTATED part: with rot_dim > 0 every query head has rot_dim more coordinates behind its `dim` unrotated ones, the down-projection
     rot_dim more rows behind the latent -- one key part shared by all heads -- and both are turned by the position (neighbouring pairs
     (2i, 2i + 1), angle p * rot_base^(-2i / rot_dim)); score = (q_plain . k_plain + q_rot . k_rot) * scale.  The cached row is [latent |
     rotated key part]; the up-projections are widened on the host (identity columns in uk, zeros in uv), so the kernels see one latent of
-    rank + rot_dim numbers and heads of dim + rot_dim.
+    rank + rot_dim numbers and heads of dim + rot_dim.  rot_layout "half" pairs coordinate i with i + rot_dim / 2 instead of its
+    neighbour; rot_scaling {factor, original, fast, slow} rescales the frequencies for contexts longer than `original` (scaled_frequencies).
     Tensors under `prefix`: q (heads*(dim+rot_dim), width), dkv (rank+rot_dim, width), dkv.norm (rank), uk (heads*dim, rank), uv (heads*vdim,
     rank), sink (heads), g (heads, width), o (width, heads*vdim).  q | dkv | g are fused into one product."""
 
-    def __init__(self, name, width, heads, dim, vdim, rank, scale, eps, sink=True, gate=True, rot_dim=0, rot_base=10000.0, window=0):
-        if rot_dim % 2 or rot_dim < 0 or window < 0:
-            raise ZLError("latent attention: the rotated part is even, the window not negative")
+    def __init__(self, name, width, heads, dim, vdim, rank, scale, eps, sink=True, gate=True, rot_dim=0, rot_base=10000.0, window=0,
+                 rot_layout="pairs", rot_scaling=None):
+        if rot_dim % 2 or rot_dim < 0 or window < 0 or rot_layout not in ("pairs", "half"):
+            raise ZLError("latent attention: the rotated part is even, the window not negative, the layout pairs or half")
+        self.rot_layout, self.rot_scaling, self.rot_gain = rot_layout, (dict(rot_scaling) if rot_scaling else None), 1.0
         self.name, self.width, self.heads, self.dim, self.vdim, self.rank = name, width, heads, dim, vdim, rank
         self.scale, self.eps, self.has_sink, self.has_gate = float(scale), float(eps), sink, gate
         self.rot, self.rot_base, self.window = int(rot_dim), float(rot_base), int(window)
@@ -77,8 +96,13 @@ class LatentAttention:
         self.w_uk, self.w_uv = self._widen(_mat(get, prefix + "uk", (H * d, r), dtype, device), _mat(get, prefix + "uv", (H * v, r), dtype, device))
         self.sink = _vec(get, prefix + "sink", H, device) if self.has_sink else None
         self.w_o = _mat(get, prefix + "o", (W, H * v), dtype, device)
-        self.freq = rotary_frequencies(self.rot, self.rot_base, 1.0, device) if self.rot else None
+        self._tables(device)
         return self
+
+    def _tables(self, device):
+        self.freq = None
+        if self.rot:
+            self.freq, self.rot_gain = scaled_frequencies(self.rot, self.rot_base, self.rot_scaling, device)
 
     def init_random(self, gen, dtype, device):
         H, d, v, r, W = self.heads, self.dim, self.vdim, self.rank, self.width
@@ -87,7 +111,7 @@ class LatentAttention:
         self.w_uk, self.w_uv = self._widen(_rand(gen, (H * d, r), r ** -0.5, dtype, device), _rand(gen, (H * v, r), r ** -0.5, dtype, device))
         self.sink = torch.zeros(H, device=device) if self.has_sink else None
         self.w_o = _rand(gen, (W, H * v), (H * v) ** -0.5, dtype, device)
-        self.freq = rotary_frequencies(self.rot, self.rot_base, 1.0, device) if self.rot else None
+        self._tables(device)
         return self
 
     def bind(self, cache, dtype):
@@ -99,8 +123,9 @@ class LatentAttention:
     def forward(self, h, batch):
         H, d, r = self.heads, self.qdim, self.row                                # (sizes as the kernels see them: with the rotated part)
         proj = seqops.gemm_nt(h, self.w_in)                                       # fp32 [q | latent, rotated key part | gate]
-        seqops.latent_store(proj, H * d, self.dkv_norm, self.eps, self.rank, batch, self.cache, rot=self.rot, freq=self.freq, interleaved=True,
-                            q_col0=0, heads=H, qdim=d)
+        self.side = (proj, self.side_col0)
+        seqops.latent_store(proj, H * d, self.dkv_norm, self.eps, self.rank, batch, self.cache, rot=self.rot, freq=self.freq,
+                            interleaved=self.rot_layout == "pairs", q_col0=0, heads=H, qdim=d, rot_gain=self.rot_gain)
         gate = proj if self.has_gate else None
         prompt = batch.n_ctx > 0 and self.prompt_kernel and h.dtype == torch.bfloat16 and max(d, self.vdim) <= 256
         a = torch.empty((batch.n_tok, H * self.vdim), dtype=h.dtype, device=h.device)
@@ -208,7 +233,44 @@ def rotary_frequencies(n_rot, base, divide=1.0, device="cpu"):
     return (torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / n_rot) / float(divide)).to(torch.float32).to(device)
 
 
-class WindowAttention:
+def scaled_frequencies(n_rot, base, scaling=None, device="cpu"):
+    """(frequencies fp32 (n_rot / 2), gain) of a rotation whose frequencies are rescaled for contexts longer than the `original` one
+    (scaling = {factor, original, fast, slow}; None: the plain frequencies and gain 1).  A pair that turns more than `fast` times over
+    `original` positions keeps its frequency f_i = base^(-2i / n_rot), one that turns less than `slow` times gets f_i / factor, and
+    between the two pair indices lo = floor(index(fast)), hi = ceil(index(slow)) -- index(t) = n_rot ln(original / (2 pi t)) / (2 ln base),
+    clamped to the head -- the two are blended linearly in i.  cos and sin are multiplied by the gain 0.1 ln(factor) + 1.  Worked out in
+    float64, rounded once."""
+    if not scaling:
+        return rotary_frequencies(n_rot, base, 1.0, device), 1.0
+    factor, original = float(scaling["factor"]), float(scaling["original"])
+
+    def index(turns):
+        return n_rot * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+    lo = max(math.floor(index(float(scaling["fast"]))), 0)
+    hi = min(math.ceil(index(float(scaling["slow"]))), n_rot - 1)
+    i = torch.arange(n_rot // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / n_rot)
+    ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+    return (f / factor * ramp + f * (1.0 - ramp)).to(torch.float32).to(device), 0.1 * math.log(factor) + 1.0
+
+
+def distance_bias_table(rel, far, longest, device):
+    """The bias of every distance 0 .. L - 1 from a table `rel` (rows, heads) of bucketed distances: the first rows // 2 distances have a
+    row each, larger ones share the other rows on a logarithmic scale that reaches the last row at the distance `far`
+    (row = half + floor(ln(n / half) / ln(far / half) * (rows - half)), at most rows - 1).  Returns fp32 (heads, L), L = far + 1 -- every
+    distance from `far` on has the last row, the kernels clamp -- or `longest` when no query ever looks that far."""
+    rows, heads = rel.shape
+    half = rows // 2
+    if half < 1 or far <= half:
+        raise ZLError("distance bias: the table needs two rows or more and a largest distance beyond its exact half")
+    L = int(far) + 1 if longest <= 0 else min(int(far) + 1, int(longest))
+    n = torch.arange(L, dtype=torch.float64)
+    big = half + torch.floor(torch.log(torch.clamp(n, min=1.0) / half) / math.log(far / half) * (rows - half)).to(torch.int64)
+    row = torch.where(n < half, n.to(torch.int64), torch.clamp(big, max=rows - 1))
+    return rel.to(torch.float32)[row.to(rel.device)].t().contiguous().to(device)
+
+
+class WindowAttention(SideRows):
     """Softmax attention with grouped key / value heads over a paged cache: rotary positions on the first `rot_dims` coordinates of every
     query and key head (pairs i, i + rot_dims / 2; every frequency divided by `rot_scaling`), queries and keys divided by their root mean
     square afterwards (qk_norm), a sliding window of `window` positions (0: none), optionally
@@ -223,13 +285,28 @@ class WindowAttention:
       * the sequence's first keep_first keys visible behind the window, at their true positions,
       * a learned sink per head in the softmax denominator (tensor `sink`; no key, no value, not scaled),
       * values blended with ANOTHER such layer's values of the same token before they are cached, v <- (1 - lam) v + lam v_other with lam
-        the scalar tensor `vmix` (v_mix_source: that layer's WindowAttention, which ran earlier in the same step).
+        the scalar tensor `vmix` (v_mix_source: that layer's WindowAttention, which ran earlier in the same step),
+      * a weight on the query / key norm shared by the heads (norm_weight; tensors q.norm, k.norm (dim)), a factor on the scores per head
+        (head_scale; tensor `temp`), scores capped by softcap * tanh(. / softcap), a learned bias by the distance between query and key
+        added after the cap (rel_far > 0; tensor `rel` (rows, heads), see distance_bias_table),
+      * queries that only see the keys of their own chunk of `chunk` positions, chunks counted from position 0 of the sequence,
+      * weights that are no softmax: weights="sigmoid" gives every visible key sigmoid(score + offset_h) (tensor `pb` (heads)), not
+        normalised over the keys.
     Tensors under `prefix`: q (heads*dim, width), k (kv_heads*dim, width), v (kv_heads*vdim, width), talk (heads, heads), g (heads*vdim, width),
     o (width, heads*vdim).  q | k | v | g are one product."""
 
     def __init__(self, name, width, heads, kv_heads, dim, vdim, scale, window, rot_dims, rot_base, rot_scaling, eps, qk_norm=True,
                  rotate_values=True, talk=True, gate=True, kv_source=None, rope_interleaved=False, bias=False, conv_taps=0, keep_first=0,
-                 sink=False, v_mix=False, v_mix_source=None):
+                 sink=False, v_mix=False, v_mix_source=None, norm_weight=False, head_scale=False, softcap=0.0, rel_far=0, chunk=0,
+                 weights="softmax"):
+        if weights not in ("softmax", "sigmoid") or (weights == "sigmoid" and (sink or talk)) or (chunk and keep_first) or chunk < 0:
+            raise ZLError("attention: sigmoid weights have no sink and no mixing; chunks keep no first keys")
+        if norm_weight and not qk_norm:
+            raise ZLError("attention: a norm weight needs the query / key norm")
+        self.norm_weight, self.has_head_scale, self.softcap, self.rel_far, self.chunk = bool(norm_weight), bool(head_scale), float(softcap or 0.0), \
+            int(rel_far or 0), int(chunk or 0)
+        self.sigmoid = weights == "sigmoid"
+        self.q_norm_w = self.k_norm_w = self.temp = self.rel = self.offset = self.form = None
         if heads % kv_heads or rot_dims % 2 or rot_dims > dim or (rotate_values and vdim % 2):
             raise ZLError("attention: heads must divide by kv_heads, rotated sizes must be even and fit the head")
         if kv_source is not None and (kv_source.kv_heads, kv_source.dim, kv_source.vdim) != (kv_heads, dim, vdim):
@@ -260,6 +337,24 @@ class WindowAttention:
     def _tables(self, device):
         self.qk_freq = rotary_frequencies(self.rot_dims, self.rot_base, self.rot_scaling, device) if self.rot_dims else None
         self.v_freq = rotary_frequencies(self.vdim, self.rot_base, 1.0, device) if self.rotate_values else None
+        self.form = None
+        if self.has_head_scale or self.softcap > 0 or self.rel is not None or self.chunk or self.sigmoid:
+            self.form = seqops.score_form(self.heads, self.temp, self.softcap, self.rel, self.offset, self.chunk, self.sigmoid)
+
+    def _load_form(self, get, prefix, device):
+        d, H = self.dim, self.heads
+        if self.norm_weight:
+            self.q_norm_w, self.k_norm_w = _vec(get, prefix + "q.norm", d, device), _vec(get, prefix + "k.norm", d, device)
+        if self.has_head_scale:
+            self.temp = _vec(get, prefix + "temp", H, device)
+        if self.rel_far:
+            rel = get(prefix + "rel")
+            if rel.dim() != 2 or rel.shape[1] != H:
+                raise ZLError(f"tensor {prefix}rel: shape {tuple(rel.shape)}, expected (rows, {H})")
+            longest = min(x for x in (self.chunk, self.window) if x > 0) if (self.chunk or self.window) else 0
+            self.rel = distance_bias_table(rel, self.rel_far, longest, device)
+        if self.sigmoid:
+            self.offset = _vec(get, prefix + "pb", H, device)
 
     def load(self, get, prefix, dtype, device):
         H, G, d, v, W = self.heads, self.kv_heads, self.dim, self.vdim, self.width
@@ -282,6 +377,7 @@ class WindowAttention:
         self.sink = _vec(get, prefix + "sink", H, device) if self.has_sink else None
         if self.v_mix:
             self.vmix_lambda = float(_vec(get, prefix + "vmix", 1, device)[0])
+        self._load_form(get, prefix, device)
         self._tables(device)
         return self
 
@@ -299,6 +395,16 @@ class WindowAttention:
             self.conv_w = torch.ones((C, 1), device=device)
         self.sink = torch.zeros(H, device=device) if self.has_sink else None
         self.vmix_lambda = 0.5 if self.v_mix else 0.0
+        d = self.dim
+        if self.norm_weight:
+            self.q_norm_w, self.k_norm_w = 1.0 + 0.1 * torch.randn(d, generator=gen, device=device), 1.0 + 0.1 * torch.randn(d, generator=gen, device=device)
+        if self.has_head_scale:
+            self.temp = 1.0 + 0.1 * torch.randn(H, generator=gen, device=device)
+        if self.rel_far:
+            longest = min(x for x in (self.chunk, self.window) if x > 0) if (self.chunk or self.window) else 0
+            self.rel = distance_bias_table(0.5 * torch.randn(32, H, generator=gen, device=device), max(self.rel_far, 17), longest, device)
+        if self.sigmoid:
+            self.offset = -2.0 + 0.1 * torch.randn(H, generator=gen, device=device)
         self._tables(device)
         return self
 
@@ -319,6 +425,7 @@ class WindowAttention:
         k0, v0, g0, _ = self._cols()
         own = self.kv_source is None
         proj = seqops.gemm_nt(h, self.w_in)                                       # fp32 [q | k | v | gate]
+        self.side = (proj, self.side_col0)
         # biases and the short convolution give a second buffer [q | k | v] (the gate stays in proj); otherwise q is rotated inside proj
         qkv = seqops.short_conv(proj, 0, self.conv_w, self.in_bias, self.tail, batch) if self.conv_w is not None else proj
         blend = None
@@ -327,12 +434,13 @@ class WindowAttention:
             blend = (src, col, self.vmix_lambda)
         self.last_values = (qkv, v0) if self.v_mix else None                      # (this step's values before blending, for a later layer)
         seqops.rope_norm_store(qkv, 0, k0, v0, H, G, d, v, self.qk_freq, self.rot_dims, self.v_freq, self.eps, self.qk_norm, batch,
-                               self.k_cache if own else None, self.v_cache if own else None, interleaved=self.interleaved, vmix=blend)
+                               self.k_cache if own else None, self.v_cache if own else None, interleaved=self.interleaved, vmix=blend,
+                               q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w)
         acc, ml, n_splits = seqops.window_attention(qkv, 0, self.k_cache, self.v_cache, batch, self.scale, self.window, H, G, d, v,
                                                     all_kv=self.has_talk, mfma=self.prompt_kernel, n_splits=self.n_splits,
-                                                    keep_first=self.keep_first)
+                                                    keep_first=self.keep_first, form=self.form)
         a = seqops.head_mix_gate(acc, ml, n_splits, self.talk, self.v_freq, proj if self.has_gate else None, g0, batch, H, G, v, h.dtype,
-                                 sink=self.sink)
+                                 sink=self.sink, plain_sum=self.sigmoid)
         return seqops.gemm_nt(a, self.w_o)
 
 
@@ -436,6 +544,35 @@ class GatedLinearAttention:
         return seqops.gemm_nt(a, self.w_o)
 
 
+class PlainFF(SideRows):
+    """Dense feed-forward down(act(up h)) without biases and without a gate; act: "relu2" (the square of relu), "gelu_tanh" or "silu".
+    Tensors under `prefix`: up (ff, width), down (width, ff)."""
+    _side_matrix = "w_up"
+
+    def __init__(self, width, ff, act="relu2"):
+        if act not in seqops.UNARY_ACTS:
+            raise ZLError(f"feed-forward: unknown activation {act!r}")
+        self.width, self.ff, self.act = width, ff, act
+
+    def load(self, get, prefix, dtype, device):
+        self.w_up = _mat(get, prefix + "up", (self.ff, self.width), dtype, device)
+        self.w_down = _mat(get, prefix + "down", (self.width, self.ff), dtype, device)
+        return self
+
+    def init_random(self, gen, dtype, device):
+        self.w_up = _rand(gen, (self.ff, self.width), self.width ** -0.5, dtype, device)
+        self.w_down = _rand(gen, (self.width, self.ff), self.ff ** -0.5, dtype, device)
+        return self
+
+    def weight_bytes(self):
+        return sum(t.numel() * t.element_size() for t in (self.w_up, self.w_down))
+
+    def forward(self, h):
+        z = seqops.gemm_nt(h, self.w_up)                                          # fp32 [up | side rows]
+        self.side = (z, self.side_col0)
+        return seqops.gemm_nt(seqops.unary_act(z, h.dtype, kind=self.act, cols=self.ff), self.w_down)
+
+
 class GatedFF:
     """Dense gated feed-forward down(act(gate h) * (up h)) without biases; act: "gelu_tanh" (the tanh form) or "silu".
     Tensors under `prefix`: gate, up (ff, width), down (width, ff).  gate | up are one product."""
@@ -518,13 +655,14 @@ class RoutedExpertsFF:
     """Mixture of gated feed-forward experts, down(silu(gate h) * (up h)), without biases.  The router gives one logit per expert and per
     IDENTITY output (the last `identity` of its outputs: their "expert" returns h itself); probabilities = softmax over all outputs; an
     output is chosen by probability + `correction`, within the `keep` best of `groups` equal groups of neighbouring outputs (a group scores
-    by its best member); the `top` chosen outputs are weighted by their plain probabilities (renormalised only if `renorm`).
+    by its best member); the `top` chosen outputs are weighted by their plain probabilities (renormalised only if `renorm`), times
+    `weight_scale`.
     Tensors under `prefix`: router (experts + identity, width), correction (experts + identity), e<j>.gate / e<j>.up (ff, width),
     e<j>.down (width, ff).  Gate and up rows of all experts are stacked in blocks of 16 (16 gate rows, their 16 up rows), so that the grouped
     product's epilogue finishes the activation."""
 
     def __init__(self, width, ff, experts, top, identity=0, groups=1, keep=1, correction=True, renorm=False, score="softmax", group_top=1,
-                 renorm_eps=0.0, act="silu", act_alpha=1.0, limit=0.0):
+                 renorm_eps=0.0, act="silu", act_alpha=1.0, limit=0.0, weight_scale=1.0):
         """score: "softmax" over all outputs or "sigmoid" of each logit; group_top: a group scores by the sum of its group_top best choice
         scores; act: "silu" -- silu(gate) up --, or "swish_clamp" -- g sigmoid(act_alpha g) (u + 1) with g = min(gate, limit),
         u = clamp(up, -limit, limit)"""
@@ -532,6 +670,7 @@ class RoutedExpertsFF:
             raise ZLError("experts: unknown score function or activation")
         self.score, self.group_top, self.renorm_eps, self.act, self.act_alpha, self.limit = score, int(group_top), float(renorm_eps), act, \
             float(act_alpha), float(limit)
+        self.weight_scale = float(weight_scale)
         total = experts + identity
         if groups < 1 or total % groups or not 1 <= keep <= groups or top > keep * (total // groups):
             raise ZLError("experts: groups must divide the router outputs, and the kept groups must hold `top` outputs")
@@ -574,7 +713,7 @@ class RoutedExpertsFF:
     def forward(self, h):
         logits = seqops.gemm_nt(h, self.w_router)                                 # fp32 sums of the products
         ids, weights = seqops.moe_route(logits, self.correction, self.groups, self.keep, self.top, self.renorm, score=self.score,
-                                        group_top=self.group_top, renorm_eps=self.renorm_eps)
+                                        group_top=self.group_top, renorm_eps=self.renorm_eps, weight_scale=self.weight_scale)
         sorted_tok, slot_pos, tiles, max_tiles, sorted_exp, tm = seqops.moe_align(ids, self.experts, self.tile_m)
         n_slots = ids.numel()
         few = sorted_exp if n_slots <= self.few_rows else None                    # decode steps: weight rows streamed per (row, column)

@@ -25,6 +25,7 @@ def _ensure_builtin():
     from . import tupitar  # noqa: F401  (registers itself)
     from . import retotar  # noqa: F401
     from . import gutivik  # noqa: F401
+    from . import gaparax  # noqa: F401
     from . import llama    # noqa: F401
 
 

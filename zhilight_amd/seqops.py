@@ -20,7 +20,8 @@ SYMBOLS = ["zls_version", "zls_gemm_nt", "zls_embed", "zls_token_shift", "zls_ad
            "zls_conv_silu", "zls_conv_tail_update", "zls_ssm_scan", "zls_ssm_scan_workspace_bytes", "zls_gated_group_norm", "zls_layer_norm",
            "zls_add_layer_norm", "zls_rope_norm_store", "zls_window_attention", "zls_window_attention_prompt", "zls_head_mix_gate", "zls_decay_scan", "zls_exp_gates",
            "zls_linear_attn_finish", "zls_moe_route", "zls_moe_align", "zls_gemm_nt_grouped", "zls_silu_mul", "zls_moe_combine", "zls_rms_norm",
-           "zls_add_rms_norm", "zls_scale_softcap", "zls_act_mul", "zls_short_conv", "zls_short_conv_tail", "zls_lowrank_decay", "zls_latent_rope_store"]
+           "zls_add_rms_norm", "zls_scale_softcap", "zls_act_mul", "zls_short_conv", "zls_short_conv_tail", "zls_lowrank_decay", "zls_latent_rope_store",
+           "zls_streams_norm", "zls_streams_update", "zls_unary_act"]
 _STATUS = {-1: "invalid argument (null pointer / non-positive size)", -2: "shape not supported", -3: "dtype not supported",
            -4: "exceeds a hardware limit"}
 
@@ -30,6 +31,12 @@ class Batch(C.Structure):
     _fields_ = [("n_seq", C.c_int32), ("n_tok", C.c_int32), ("max_pages", C.c_int32), ("page_size", C.c_int32), ("max_count", C.c_int32),
                 ("reserved", C.c_int32), ("seq_start", C.c_void_p), ("seq_pos0", C.c_void_p), ("seq_slot", C.c_void_p),
                 ("tok_seq", C.c_void_p), ("page_table", C.c_void_p)]
+
+
+class ScoreForm(C.Structure):
+    """zls_score_form_t"""
+    _fields_ = [("head_scale", C.c_void_p), ("softcap", C.c_float), ("bias", C.c_void_p), ("bias_rows", C.c_int32), ("offset", C.c_void_p),
+                ("chunk", C.c_int32), ("sigmoid", C.c_int32)]
 
 
 _lib = None
@@ -245,9 +252,10 @@ def polynorm(z, coef, eps, dtype):
     return out
 
 
-def latent_store(proj, col0, weight, eps, rank, batch, cache, rot=0, freq=None, interleaved=True, q_col0=0, heads=0, qdim=0):
+def latent_store(proj, col0, weight, eps, rank, batch, cache, rot=0, freq=None, interleaved=True, q_col0=0, heads=0, qdim=0, rot_gain=1.0):
     """normed latent -> the tokens' cache rows; rot > 0: the `rot` columns behind the latent (one key part for all heads) are turned by the
-    position and stored behind it, and the last rot of the qdim coordinates of every query head (from q_col0) are turned in place"""
+    position and stored behind it, and the last rot of the qdim coordinates of every query head (from q_col0) are turned in place; cos and
+    sin times rot_gain"""
     _cuda(proj, weight, cache, freq)
     _f32(proj, weight, freq)
     if cache.dim() != 3 or cache.shape[1] != batch.c.page_size or cache.shape[2] != rank + rot or weight.numel() != rank:
@@ -255,7 +263,7 @@ def latent_store(proj, col0, weight, eps, rank, batch, cache, rot=0, freq=None, 
     if rot and (freq is None or freq.numel() != rot // 2):
         raise ZLError("latent_store: one frequency per rotated pair")
     check(lib().zls_latent_rope_store(_p(proj), _i(proj.shape[1]), _i(col0), _p(weight), _f(eps), _i(rank), _i(rot), _p(freq),
-                                      C.c_int(int(interleaved)), _i(q_col0), _i(heads), _i(qdim), batch.ref, _p(cache),
+                                      C.c_int(int(interleaved)), _i(q_col0), _i(heads), _i(qdim), _f(rot_gain), batch.ref, _p(cache),
                                       C.c_int(dt_code(cache.dtype)), _stream()), "latent_store")
 
 
@@ -427,6 +435,59 @@ def add_rms_norm(x, y, eps, next_weight=None, dtype=None, around_zero=False):
     return h2
 
 
+# ---- a residual kept as several streams ------------------------------------------------------------------------------------------------
+def streams_norm(xs, n, read_coef, weight, eps, dtype, rows=None, around_zero=False):
+    """N(sum_s read_coef[s] x_s) of the rows `rows` (None: all) in `dtype`.  xs fp32: (n_tok, n, width), or (n_tok, width) read as n equal
+    streams; read_coef fp32 (n) or None (all 1)"""
+    _cuda(xs, read_coef, weight, rows)
+    _f32(xs, read_coef, weight)
+    width = xs.shape[-1]
+    if xs.dim() == 3 and xs.shape[1] != n or (read_coef is not None and read_coef.numel() != n) or weight.numel() != width:
+        raise ZLError("streams_norm: shapes")
+    if rows is not None and rows.dtype != torch.int32:
+        raise ZLError("streams_norm: rows must be int32")
+    tok, stream = (n * width, width) if xs.dim() == 3 else (width, 0)
+    n_rows = xs.shape[0] if rows is None else rows.numel()
+    h = torch.empty((n_rows, width), dtype=dtype, device=xs.device)
+    check(lib().zls_streams_norm(_p(xs), _i(tok), _i(stream), _i(n), _p(read_coef), _p(rows), _p(weight), _f(1.0 if around_zero else 0.0),
+                                 _f(eps), _i(n_rows), _i(width), _p(h), C.c_int(dt_code(dtype)), _stream()), "streams_norm")
+    return h
+
+
+def streams_update(src, dst, n, y, mix, out_coef, gate=None, g_col0=0, gate_bias=None, next_coef=None, next_weight=None, eps=0.0, dtype=None,
+                   around_zero=False):
+    """dst_d = sum_s mix[s][d] src_s + out_coef[d] * y * sigmoid(gate[:, g_col0:] + gate_bias) for all streams at once (dst may be src; src
+    (n_tok, width) is read as n equal streams); with next_coef also returns N(sum_d next_coef[d] dst_d) in `dtype`"""
+    _cuda(src, dst, y, mix, out_coef, gate, gate_bias, next_coef, next_weight)
+    _f32(src, dst, y, mix, out_coef, gate, gate_bias, next_coef, next_weight)
+    n_tok, width = y.shape
+    if tuple(dst.shape) != (n_tok, n, width) or mix.numel() != n * n or out_coef.numel() != n or src.shape[0] != n_tok or src.shape[-1] != width \
+            or (src.dim() == 3 and src.shape[1] != n) or (gate_bias is not None and gate_bias.numel() != width):
+        raise ZLError("streams_update: shapes")
+    tok, stream = (n * width, width) if src.dim() == 3 else (width, 0)
+    h = torch.empty((n_tok, width), dtype=dtype, device=y.device) if next_coef is not None else None
+    check(lib().zls_streams_update(_p(src), _i(tok), _i(stream), _p(dst), _i(n), _p(y), _p(gate), _i(0 if gate is None else gate.stride(0)),
+                                   _i(g_col0), _p(gate_bias), _p(mix), _p(out_coef), _p(next_coef), _p(next_weight),
+                                   _f(1.0 if around_zero else 0.0), _f(eps), _i(n_tok), _i(width), _p(h),
+                                   C.c_int(dt_code(dtype) if h is not None else BF16), _stream()), "streams_update")
+    return h
+
+
+UNARY_ACTS = {"relu2": 0, "gelu_tanh": 1, "silu": 2}
+
+
+def unary_act(z, dtype, kind="relu2", cols=None):
+    """act(z[:, :cols]) of fp32 rows in `dtype`; see UNARY_ACTS"""
+    _f32(z)
+    if z.dim() != 2 or z.stride(1) != 1 or not z.is_cuda:
+        raise ZLError("unary_act: z must be a device matrix with unit column stride")
+    cols = z.shape[1] if cols is None else cols
+    out = torch.empty((z.shape[0], cols), dtype=dtype, device=z.device)
+    check(lib().zls_unary_act(_p(z), _i(z.stride(0)), _i(z.shape[0]), _i(cols), C.c_int(UNARY_ACTS[kind]), _p(out), C.c_int(dt_code(dtype)),
+                              _stream()), "unary_act")
+    return out
+
+
 def scale_softcap(z, scale, cap):
     """z <- cap * tanh(z * scale / cap) in place (cap <= 0: z * scale); fp32"""
     _cuda(z)
@@ -437,11 +498,15 @@ def scale_softcap(z, scale, cap):
 
 # ---- softmax attention over paged keys and values -------------------------------------------------------------------------------------------
 def rope_norm_store(proj, q_col0, k_col0, v_col0, heads, kv_heads, dim, vdim, qk_freq, rot_dims, v_freq, eps, qk_norm, batch, k_cache, v_cache,
-                    interleaved=False, vmix=None):
+                    interleaved=False, vmix=None, q_norm_w=None, k_norm_w=None):
     """rotate / norm the queries in place in proj; rotate / norm the keys and turn the values into the paged planes (None: queries only).
-    interleaved: rotated pairs are neighbours (2i, 2i + 1).  vmix = (src, col0, lam): values <- (1 - lam) values + lam src[t][col0 ..]"""
-    _cuda(proj, qk_freq, v_freq, k_cache, v_cache)
-    _f32(proj, qk_freq, v_freq)
+    interleaved: rotated pairs are neighbours (2i, 2i + 1).  vmix = (src, col0, lam): values <- (1 - lam) values + lam src[t][col0 ..].
+    q_norm_w / k_norm_w: fp32 (dim) weights of the norm, shared by the heads"""
+    _cuda(proj, qk_freq, v_freq, k_cache, v_cache, q_norm_w, k_norm_w)
+    _f32(proj, qk_freq, v_freq, q_norm_w, k_norm_w)
+    for t in (q_norm_w, k_norm_w):
+        if t is not None and (t.numel() != dim or not qk_norm):
+            raise ZLError("rope_norm_store: a norm weight has one number per coordinate of a head")
     vsrc, vcol, vlam = vmix if vmix is not None else (None, 0, 0.0)
     if vsrc is not None and (vsrc.dtype != torch.float32 or vsrc.dim() != 2 or vsrc.stride(1) != 1 or vsrc.shape[0] != batch.n_tok):
         raise ZLError("rope_norm_store: the blended values are fp32 rows, one per token")
@@ -455,12 +520,28 @@ def rope_norm_store(proj, q_col0, k_col0, v_col0, heads, kv_heads, dim, vdim, qk
     code = dt_code(k_cache.dtype) if k_cache is not None else F32
     check(lib().zls_rope_norm_store(_p(proj), _i(proj.shape[1]), _i(q_col0), _i(k_col0), _i(v_col0), _i(heads), _i(kv_heads), _i(dim), _i(vdim),
                                     _p(qk_freq), _i(rot_dims), _p(v_freq), _f(eps), C.c_int(int(qk_norm)), C.c_int(int(interleaved)), _p(vsrc),
-                                    _i(0 if vsrc is None else vsrc.stride(0)), _i(vcol), _f(vlam), batch.ref, _p(k_cache), _p(v_cache),
+                                    _i(0 if vsrc is None else vsrc.stride(0)), _i(vcol), _f(vlam), _p(q_norm_w), _p(k_norm_w), batch.ref, _p(k_cache), _p(v_cache),
                                     C.c_int(code), _stream()), "rope_norm_store")
 
 
+def score_form(heads, head_scale=None, softcap=0.0, bias=None, offset=None, chunk=0, sigmoid=False):
+    """The optional score form of window_attention: per-head factor (heads), tanh cap, distance bias fp32 (heads, rows) -- row min(p - j,
+    rows - 1) --, chunked visibility, sigmoid weights with a per-head offset.  Returns an object that keeps the tensors alive."""
+    _cuda(head_scale, bias, offset)
+    _f32(head_scale, bias, offset)
+    for t in (head_scale, offset):
+        if t is not None and t.numel() != heads:
+            raise ZLError("score_form: one number per head")
+    if bias is not None and (bias.dim() != 2 or bias.shape[0] != heads):
+        raise ZLError("score_form: the distance bias is (heads, rows)")
+    f = ScoreForm(0 if head_scale is None else head_scale.data_ptr(), float(softcap or 0.0), 0 if bias is None else bias.data_ptr(),
+                  0 if bias is None else bias.shape[1], 0 if offset is None else offset.data_ptr(), int(chunk), int(bool(sigmoid)))
+    f.keep = (head_scale, bias, offset)
+    return f
+
+
 def window_attention(q, q_col0, k_cache, v_cache, batch, scale, window, heads, kv_heads, dim, vdim, all_kv, mfma=True, n_splits=None,
-                     keep_first=0):
+                     keep_first=0, form=None):
     """Every query head's softmax weights applied to its own (all_kv False) or every kv head's values.  Returns (acc, ml, n_splits) for
     head_mix_gate: fp32 partial sums (n_tok, heads, n_splits, nv) and their (maximum, weight sum).  bf16 portions run on the matrix cores
     when the sizes allow (mfma=False: everything on the plain kernel); single tokens are split over their window's pages."""
@@ -474,6 +555,9 @@ def window_attention(q, q_col0, k_cache, v_cache, batch, scale, window, heads, k
     plain_tokens = batch.n_single if prompt else batch.n_tok
     # the pages a window can touch, and enough workgroups to fill the chip (256 CUs, a few per CU) when few tokens take the plain kernel
     span = min(batch.max_ctx, window) if window > 0 else batch.max_ctx
+    if form is not None and form.chunk > 0:
+        span = min(span, form.chunk)                                 # (a chunk's keys: at most chunk positions, wherever they start in a page)
+    fref = C.byref(form) if form is not None else None
     keep_first = int(keep_first) if window > 0 else 0                # (keys 0 .. keep_first - 1 stay visible behind the window)
     pages = min((span + ps - 2) // ps + 1 + (keep_first + ps - 1) // ps, (batch.max_ctx + ps - 1) // ps)
     if n_splits is None:
@@ -486,15 +570,15 @@ def window_attention(q, q_col0, k_cache, v_cache, batch, scale, window, heads, k
     if prompt:
         check(lib().zls_window_attention_prompt(_p(q), _i(q.shape[1]), _i(q_col0), _p(k_cache), _p(v_cache), batch.ref, _p(batch.q_tiles),
                                                 _i(batch.n_q_tiles), _f(scale), _i(window), _i(keep_first), _i(heads), _i(kv_heads), _i(dim), _i(vdim),
-                                                C.c_int(int(all_kv)), _p(acc), _p(ml), _i(n_splits), code, _stream()), "window_attention_prompt")
+                                                C.c_int(int(all_kv)), _p(acc), _p(ml), _i(n_splits), fref, code, _stream()), "window_attention_prompt")
     if plain_tokens:
         check(lib().zls_window_attention(_p(q), _i(q.shape[1]), _i(q_col0), _p(k_cache), _p(v_cache), batch.ref, _f(scale), _i(window), _i(keep_first), _i(heads),
                                          _i(kv_heads), _i(dim), _i(vdim), C.c_int(int(all_kv)), _p(acc), _p(ml), _i(n_splits), _i(per),
-                                         C.c_int(int(prompt)), code, _stream()), "window_attention")
+                                         C.c_int(int(prompt)), fref, code, _stream()), "window_attention")
     return acc, ml, n_splits
 
 
-def head_mix_gate(acc, ml, n_splits, talk, v_freq, gate, g_col0, batch, heads, kv_heads, vdim, dtype, sink=None):
+def head_mix_gate(acc, ml, n_splits, talk, v_freq, gate, g_col0, batch, heads, kv_heads, vdim, dtype, sink=None, plain_sum=False):
     _cuda(acc, ml, talk, v_freq, gate, sink)
     _f32(acc, ml, talk, v_freq, gate, sink)
     if sink is not None and sink.numel() != heads:
@@ -505,8 +589,8 @@ def head_mix_gate(acc, ml, n_splits, talk, v_freq, gate, g_col0, batch, heads, k
         raise ZLError("head_mix_gate: acc / ml do not fit")
     out = torch.empty((batch.n_tok, heads * vdim), dtype=dtype, device=acc.device)
     check(lib().zls_head_mix_gate(_p(acc), _p(ml), _i(n_splits), _p(talk), _p(v_freq), _p(gate), _i(0 if gate is None else gate.shape[1]),
-                                  _i(g_col0), _p(sink), batch.ref, _i(heads), _i(kv_heads), _i(vdim), _p(out), C.c_int(dt_code(dtype)), _stream()),
-          "head_mix_gate")
+                                  _i(g_col0), _p(sink), C.c_int(int(plain_sum)), batch.ref, _i(heads), _i(kv_heads), _i(vdim), _p(out), C.c_int(dt_code(dtype)),
+                                  _stream()), "head_mix_gate")
     return out
 
 
@@ -576,7 +660,7 @@ MOE_TILE = 64           # rows of an expert's tile in the grouped products; 128 
 MOE_BIG_SHARE = 256
 
 
-def moe_route(logits, correction, groups, keep, top, renorm=False, score="softmax", group_top=1, renorm_eps=0.0):
+def moe_route(logits, correction, groups, keep, top, renorm=False, score="softmax", group_top=1, renorm_eps=0.0, weight_scale=1.0):
     _cuda(logits, correction)
     _f32(logits, correction)
     n_tok, n_out = logits.shape
@@ -587,7 +671,8 @@ def moe_route(logits, correction, groups, keep, top, renorm=False, score="softma
     if score not in ("softmax", "sigmoid"):
         raise ZLError("moe_route: scores are softmax or sigmoid")
     check(lib().zls_moe_route(_p(logits), _i(n_tok), _i(n_out), _p(correction), _i(groups), _i(keep), _i(top), C.c_int(int(renorm)),
-                              C.c_int(1 if score == "sigmoid" else 0), _i(group_top), _f(renorm_eps), _p(ids), _p(weights), _stream()), "moe_route")
+                              C.c_int(1 if score == "sigmoid" else 0), _i(group_top), _f(renorm_eps), _f(weight_scale), _p(ids), _p(weights), _stream()),
+          "moe_route")
     return ids, weights
 
 
