@@ -55,6 +55,24 @@ def chunk_visible(T, size):
 
 
 # ---- sigmoid attention -----------------------------------------------------------------------------------------------------------------
+def sigmoid_attention(q, k, v, scale, temp, cap, bias, vis, offset):
+    """q (T, H, d), k (T, G, d), v (T, G, e); head a reads kv head a // (H / G); score = q.k * scale * temp[a], capped by cap * tanh(. / cap)
+    when cap > 0, plus bias[a] (T, T); the weight of a visible key is sigmoid(score + offset[a]), every key on its own"""
+    T, H, _ = q.shape
+    G = k.shape[1]
+    out = torch.zeros(T, H, v.shape[2], dtype=F64)
+    for a in range(H):
+        g = a // (H // G)
+        s = (q[:, a] @ k[:, g].T) * scale * temp[a]
+        if cap > 0:
+            s = cap * torch.tanh(s / cap)
+        if bias is not None:
+            s = s + bias[a]
+        w = torch.where(vis, torch.sigmoid(s + offset[a]), torch.zeros((), dtype=F64))
+        out[:, a] = w @ v[:, g]
+    return out
+
+
 def sigmoid_attention_mixer(h, weights, p, m, eps):
     """grouped attention whose weights are sigmoids, not a softmax: q and k normed per head, score scaled, multiplied by a number per head,
     capped by tanh, a distance bias added, then sigmoid(score + offset_h) for every visible key of the query's chunk; the heads' sums are
@@ -67,15 +85,7 @@ def sigmoid_attention_mixer(h, weights, p, m, eps):
     temp, offset, cap = _w(weights, p + "temp"), _w(weights, p + "pb"), float(m.get("softcap") or 0.0)
     bias = distance_bias(T, _w(weights, p + "rel"), m["bias_max"])
     vis = chunk_visible(T, int((m.get("mask") or {}).get("size", 0)))
-    out = torch.zeros(T, H, e, dtype=F64)
-    for a in range(H):
-        g = a // (H // G)
-        s = (q[:, a] @ k[:, g].T) * m["scale"] * temp[a]
-        if cap > 0:
-            s = cap * torch.tanh(s / cap)
-        s = s + bias[a]
-        w = torch.where(vis, torch.sigmoid(s + offset[a]), torch.zeros((), dtype=F64))
-        out[:, a] = w @ v[:, g]
+    out = sigmoid_attention(q, k, v, m["scale"], temp, cap, bias, vis, offset)
     gate = torch.sigmoid(h @ _w(weights, p + "g").T)
     return (out.reshape(T, H * e) * gate) @ _w(weights, p + "o").T
 
@@ -148,9 +158,10 @@ def dense_ff(h, weights, p):
     return (z * z) @ _w(weights, p + "down").T
 
 
-def route(h, weights, p, r):
+def route(h, weights, p, r, margins=None):
     """(ids (T, top), weights (T, top)): softmax over all experts; only experts of the `keep` groups with the largest best member count;
-    the `top` largest scores, weighted by score * router.scale"""
+    the `top` largest scores, weighted by score * router.scale.  margins (a list): receives the smallest difference of logits that decided
+    a choice -- between the last kept and the first dropped group, and between the last chosen and the first unchosen allowed expert"""
     z = h @ _w(weights, p + "router").T
     s = torch.softmax(z, -1)
     T, E = s.shape
@@ -163,12 +174,23 @@ def route(h, weights, p, r):
     kept.scatter_(1, best.topk(keep, dim=-1).indices, True)
     allowed = kept[:, :, None].expand(T, count, per).reshape(T, E)
     ids = s.masked_fill(~allowed, -1.0).topk(int(r["top"]), dim=-1).indices
+    if margins is not None:
+        gz = z.reshape(T, count, per).max(-1).values.sort(-1, descending=True).values
+        az = z.masked_fill(~allowed, -math.inf).sort(-1, descending=True).values
+        top = int(r["top"])
+        gaps = []
+        if keep < count:
+            gaps.append(gz[:, keep - 1] - gz[:, keep])
+        if top < keep * per:
+            gaps.append(az[:, top - 1] - az[:, top])
+        if gaps:
+            margins.append(float(torch.stack(gaps).min()))
     return ids, s.gather(1, ids) * float(r.get("scale", 1.0))
 
 
-def experts_ff(h, weights, p, f):
+def experts_ff(h, weights, p, f, margins=None):
     """sum over the chosen experts of weight * down(silu(gate h) * (up h))"""
-    ids, wts = route(h, weights, p, f["router"])
+    ids, wts = route(h, weights, p, f["router"], margins)
     out = torch.zeros(h.shape[0], _w(weights, p + "e0.down").shape[0], dtype=F64)
     for t in range(h.shape[0]):
         for c in range(ids.shape[1]):
@@ -193,8 +215,8 @@ def sublayer(xs, weights, p, q, fn, eps):
     return mixed + _w(weights, f"{p}hc{q}.out")[:, None, None] * y[None]
 
 
-def model(tokens, weights, cfg, keep_layers=None):
-    """logits (T, vocab) of one sequence; keep_layers: a list that receives the sum of the streams after every layer"""
+def model(tokens, weights, cfg, keep_layers=None, margins=None):
+    """logits (T, vocab) of one sequence; keep_layers: a list that receives the sum of the streams after every layer; margins: see route"""
     eps = float(cfg["norm"]["eps"])
     x = _w(weights, "embed")[torch.as_tensor(tokens, dtype=torch.long)]
     xs = x[None].repeat(int(cfg["streams"]), 1, 1)
@@ -203,8 +225,84 @@ def model(tokens, weights, cfg, keep_layers=None):
         xs = sublayer(xs, weights, p, 1, lambda h: MIXERS[l["type"]](h, weights, p + "mix.", l["mixer"], eps), eps)
         f = l.get("mlp")
         if f is not None:
-            fn = (lambda h: dense_ff(h, weights, p + "mlp.")) if f["kind"] == "dense" else (lambda h: experts_ff(h, weights, p + "mlp.", f))
+            fn = (lambda h: dense_ff(h, weights, p + "mlp.")) if f["kind"] == "dense" else (lambda h: experts_ff(h, weights, p + "mlp.", f, margins))
             xs = sublayer(xs, weights, p, 2, fn, eps)
         if keep_layers is not None:
             keep_layers.append(xs.sum(0))
     return rms_norm(xs.sum(0), _w(weights, "final.norm"), eps) @ _w(weights, "head").T
+
+
+# ---- test weights ------------------------------------------------------------------------------------------------------------------------
+def random_weights(cfg, seed=0, rel_rows=12, fixed_choice=False):
+    """every tensor the configuration asks for, bf16-representable values (both serving formats start from the same numbers).
+    fixed_choice: the routers read ONE reserved coordinate of the residual only -- coordinate 0 of the embedding holds a number whose sign
+    and size the token decides, and no sub-layer writes to it -- with evenly spaced multiples per expert, so that the order of the logits
+    is one fixed order or its reverse, with wide gaps: no choice is a close call under a rounded router input, while the chosen experts'
+    weights still follow the softmax of logits that vary with the token."""
+    g = torch.Generator().manual_seed(seed)
+    W, S = cfg["width"], cfg["streams"]
+    sd = {}
+
+    def mat(name, rows, cols, std=None):
+        sd[name] = (torch.randn(rows, cols, generator=g) * (std if std is not None else cols ** -0.5)).to(torch.bfloat16)
+
+    def vec(name, n, std=0.2, mean=0.0):
+        sd[name] = (mean + std * torch.randn(n, generator=g)).to(torch.bfloat16)
+
+    mat("embed", cfg["vocab"], W, 1.5)
+    if fixed_choice:
+        size = 2.0 + 2.0 * torch.rand(cfg["vocab"], generator=g)
+        sd["embed"][:, 0] = torch.where(torch.arange(cfg["vocab"]) % 3 == 0, -size, size).to(torch.bfloat16)
+    mat("head", cfg["vocab"], W)
+    vec("final.norm", W, 0.2, 1.0)
+    for i, l in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", l["mixer"]
+        H, d, v = m["heads"], m["dim"], m["vdim"]
+        if l["type"] == "attention":
+            G = m["kv_heads"]
+            for n, rows in (("q", H * d), ("k", G * d), ("v", G * v), ("g", H * v)):
+                mat(p + "mix." + n, rows, W)
+            vec(p + "mix.q.norm", d, 0.3, 1.0)
+            vec(p + "mix.k.norm", d, 0.3, 1.0)
+            vec(p + "mix.temp", H, 0.4, 1.5)
+            vec(p + "mix.pb", H, 0.7, -1.5)
+            sd[p + "mix.rel"] = (torch.randn(rel_rows + 2 * (i % 2), H, generator=g) * 1.2).to(torch.bfloat16)
+            mat(p + "mix.o", W, H * v)
+        else:
+            r, R = m["rot_dim"], m["kv_rank"]
+            mat(p + "mix.q", H * (d + r), W)
+            mat(p + "mix.dkv", R + r, W)
+            vec(p + "mix.dkv.norm", R, 0.2, 1.0)
+            mat(p + "mix.uk", H * d, R)
+            mat(p + "mix.uv", H * v, R)
+            vec(p + "mix.sink", H, 1.0)
+            mat(p + "mix.o", W, H * v)
+        f = l.get("mlp")
+        for q in (1, 2) if f is not None else (1,):
+            vec(f"{p}norm{q}", W, 0.2, 1.0)
+            vec(f"{p}hc{q}.in", S, 0.3, 1.0 / S)
+            vec(f"{p}hc{q}.out", S, 0.3, 0.8)
+            sd[f"{p}hc{q}.mix"] = (torch.eye(S) + 0.25 * torch.randn(S, S, generator=g)).to(torch.bfloat16)
+            mat(f"{p}rg{q}", W, W)
+            vec(f"{p}rg{q}.b", W, 0.5, 0.5)
+        if f is None:
+            continue
+        if f["kind"] == "dense":
+            mat(p + "mlp.up", f["ff"], W)
+            mat(p + "mlp.down", W, f["ff"])
+        else:
+            E, ff = f["router"]["experts"], f["expert"]["ff"]
+            mat(p + "mlp.router", E, W, 2.0 * W ** -0.5)
+            for e in range(E):
+                mat(f"{p}mlp.e{e}.gate", ff, W)
+                mat(f"{p}mlp.e{e}.up", ff, W)
+                mat(f"{p}mlp.e{e}.down", W, ff)
+            if fixed_choice:
+                r = torch.zeros(E, W)
+                r[:, 0] = 0.8 * torch.randperm(E, generator=g).double() - 0.4 * E
+                sd[p + "mlp.router"] = r.to(torch.bfloat16)
+    if fixed_choice:
+        for name, t in sd.items():
+            if name.endswith((".mix.o", ".mlp.down")) or (".mlp.e" in name and name.endswith(".down")):
+                t[:1] = 0.0
+    return sd
