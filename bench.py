@@ -19,11 +19,13 @@ fields, `roofline` (the W4A16 GEMV kernel: algorithmic bytes / HIP-event time, v
     python bench.py --mixers 1b,8b [--seq 2048]
     python bench.py --retotar 1b,8b [--seq 2048]
     python bench.py --gutivik 1b,8b [--seq 2048]
+    python bench.py --gaparax 1b,8b [--seq 2048] [--only TEXT]
 
 is a different measurement with its own JSON line: prefill / decode throughput of the ragged-step engine's latent-attention, state-space
 and hybrid stacks (zhilight_amd/tupitar.py) beside the dense bf16 Llama-shaped stack of equal width, 4 layers each, random weights;
 --retotar the same for the Retotar stacks (zhilight_amd/retotar.py) beside the Tupitar hybrid of equal width.
 --gutivik the same for the Gutivik stacks (zhilight_amd/gutivik.py) beside Retotar stacks of equal width.
+--gaparax the same for the Gaparax stacks (zhilight_amd/gaparax.py) beside Gutivik stacks of equal width.
 """
 import argparse
 import json
@@ -693,15 +695,108 @@ def bench_gutivik(args, dev):
     print(json.dumps({"metric": "gutivik_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "layers": 4, "results": results}))
 
 
+GAPARAX_BENCH_SIZES = {
+    # name: width, residual streams; attention heads / key-value heads x head size, chunk, rows and reach of the distance bias; latent attention
+    #       heads x (plain + rotated) key size, latent rank; experts x their ff, picks, groups; the dense feed-forward's ff (two matrices that
+    #       hold what the picked experts' three hold).  Head counts, sizes and experts are those of GUTIVIK_BENCH_SIZES.
+    "1b": dict(width=2048, streams=4, heads=16, kv_heads=4, dim=128, chunk=1024, rel_rows=32, far=4096, l_dim=128, l_rot=64, rank=512,
+               experts=16, ff=1360, top=4, groups=4, keep_groups=2, dense_ff=8160),
+    "8b": dict(width=4096, streams=4, heads=32, kv_heads=8, dim=128, chunk=1024, rel_rows=32, far=4096, l_dim=128, l_rot=64, rank=512,
+               experts=32, ff=2384, top=4, groups=4, keep_groups=2, dense_ff=14304),
+}
+
+
+def _measure_ragged(results, label, name, model, seq, vocab):
+    """prefill of one prompt of `seq` tokens, then single-token steps of 1 and 8 requests behind contexts of seq - 40 tokens, through
+    Engine.run_step; appends tokens/s and ms per step"""
+    from zhilight_amd.engine import Engine, Entry
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    toks = torch.randint(0, vocab, (seq,)).tolist()
+    for batch in (1, 8):
+        eng = Engine(model, max_tokens=batch * (seq + 64), max_seqs=batch)
+
+        def prefill():
+            eng.run_step([Entry("p", toks, [seq - 1])])
+            eng.release("p")
+        if batch == 1:
+            ms = timed(prefill, 3)
+            results.append(dict(model=label, size=name, phase="prefill", tokens=seq, ms=round(ms, 3), tokens_per_s=round(seq / ms * 1e3)))
+        for b in range(batch):
+            eng.run_step([Entry(f"d{b}", toks[:seq - 40], [])])
+
+        def decode():
+            eng.run_step([Entry(f"d{b}", [7], [0]) for b in range(batch)])
+        ms = timed(decode, 20)
+        results.append(dict(model=label, size=name, phase="decode", batch=batch, context=seq - 40, ms=round(ms, 3),
+                            tokens_per_s=round(batch / ms * 1e3)))
+        del eng
+
+
+def bench_gaparax(args, dev):
+    """--gaparax: prefill and decode throughput of Gaparax stacks (zhilight_amd/gaparax.py: residual streams with gated sub-layer results;
+    sigmoid attention inside chunks with a distance bias; causal latent attention with rescaled rotary frequencies and a sink; relu-squared
+    and softmax-routed expert feed-forwards) beside the closest existing model of equal width, Gutivik (windowed softmax attention, windowed
+    latent attention, sigmoid-routed experts), 4 layers each, random weights, bf16, eager launches.  One JSON line."""
+    from zhilight_amd.gaparax import GaparaxConfig, GaparaxLayerConfig, GaparaxModel
+    from zhilight_amd.gutivik import GutivikConfig, GutivikLayerConfig, GutivikModel
+    seq, vocab, results = args.seq, 32000, []
+    for name in args.gaparax.split(","):
+        z = GAPARAX_BENCH_SIZES[name]
+        mlp = dict(kind="moe", expert=dict(ff=z["ff"]), router=dict(experts=z["experts"], top=z["top"], scale=2.0,
+                                                                    groups=dict(count=z["groups"], keep=z["keep_groups"])))
+        dense = dict(kind="dense", ff=z["dense_ff"])
+        att = dict(heads=z["heads"], kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["dim"], scale=z["dim"] ** -0.5, softcap=30.0, bias_max=z["far"],
+                   mask=dict(size=z["chunk"]))
+        lat = dict(heads=z["heads"], dim=z["l_dim"], rot_dim=z["l_rot"], vdim=z["dim"], kv_rank=z["rank"], scale=(z["l_dim"] + z["l_rot"]) ** -0.5,
+                   rot=dict(dims=z["l_rot"], base=1e4, scaling=dict(factor=4.0, original=4096, fast=32.0, slow=1.0)))
+        A, L = GaparaxLayerConfig("attention", att, mlp), GaparaxLayerConfig("latent_attention", lat, mlp)
+        Ad, Ld = GaparaxLayerConfig("attention", att, dense), GaparaxLayerConfig("latent_attention", lat, dense)
+        for label, layers in (("attention x4", [A] * 4), ("latent_attention x4", [L] * 4), ("hybrid (l, a, a, l), dense / experts", [Ld, A, Ad, L])):
+            if args.only and args.only not in "gaparax " + label:
+                continue
+            model = GaparaxModel(GaparaxConfig(vocab, z["width"], z["streams"], 1e-6, 1 << 24, layers), "bfloat16", dev).init_random(1)
+            _measure_ragged(results, "gaparax " + label, name, model, seq, vocab)
+            del model
+        g = GUTIVIK_BENCH_SIZES[name]
+        gmlp = dict(kind="moe", expert=dict(ff=g["ff"], limit=7.0), router=dict(experts=g["experts"], top=g["top"],
+                                                                                groups=dict(count=g["groups"], keep=g["keep_groups"])))
+        gatt = dict(heads=g["heads"], kv_heads=g["kv_heads"], dim=g["dim"], vdim=g["dim"], scale=g["dim"] ** -0.5, conv=g["taps"],
+                    mask=dict(size=g["window"], keep_first=g["keep"]), rot=dict(dims=g["rot"], base=1e6), v_mix=True)
+        glat = dict(heads=g["heads"], dim=g["l_dim"], rot_dim=g["l_rot"], vdim=g["dim"], kv_rank=g["rank"], scale=(g["l_dim"] + g["l_rot"]) ** -0.5,
+                    mask=dict(size=g["window"]), rot=dict(dims=g["l_rot"], base=1e4))
+        GA, GL = GutivikLayerConfig("attention", gatt, gmlp), GutivikLayerConfig("latent_attention", glat, gmlp)
+        for label, layers in (("attention x4", [GA] * 4), ("latent_attention x4", [GL] * 4), ("hybrid (l, a, a, l)", [GL, GA, GA, GL])):
+            if args.only and args.only not in "gutivik " + label:
+                continue
+            model = GutivikModel(GutivikConfig(vocab, g["width"], 1e-6, 0.5, 20.0, 1 << 24, layers), "bfloat16", dev).init_random(1)
+            _measure_ragged(results, "gutivik " + label, name, model, seq, vocab)
+            del model
+    print(json.dumps({"metric": "gaparax_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "layers": 4, "results": results}))
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--gaparax", default="", metavar="SIZES",
+                    help="instead of the default workload: prefill / decode throughput of Gaparax stacks beside Gutivik stacks of equal "
+                         "width; comma-separated sizes of " + ", ".join(GAPARAX_BENCH_SIZES))
     ap.add_argument("--retotar", default="", metavar="SIZES",
                     help="instead of the default workload: prefill / decode throughput of Retotar stacks beside the Tupitar hybrid of equal "
                          "width; comma-separated sizes of " + ", ".join(RETOTAR_BENCH_SIZES))
     ap.add_argument("--gutivik", default="", metavar="SIZES",
                     help="instead of the default workload: prefill / decode throughput of Gutivik stacks beside Retotar stacks of equal "
                          "width; comma-separated sizes of " + ", ".join(GUTIVIK_BENCH_SIZES))
-    ap.add_argument("--only", default="", metavar="TEXT", help="with --gutivik: only the stacks whose label contains TEXT (e.g. for a kernel trace of one model)")
+    ap.add_argument("--only", default="", metavar="TEXT", help="with --gutivik / --gaparax: only the stacks whose label contains TEXT (e.g. for a kernel trace of one model)")
     ap.add_argument("--mixers", default="", metavar="SIZES",
                     help="instead of the default workload: prefill / decode throughput of the ragged-step engine's latent-attention + "
                          "state-space model beside the dense Llama-shaped stack of equal width; comma-separated sizes of " + ", ".join(SEQ_BENCH_SIZES))
@@ -745,6 +840,8 @@ def main():
         return bench_retotar(args, dev)
     if args.gutivik:
         return bench_gutivik(args, dev)
+    if args.gaparax:
+        return bench_gaparax(args, dev)
     from zhilight_amd import ops  # noqa: F401  (raises if the HIP library is missing)
     from zhilight_amd.llama import LLaMA, ModelConfig, QuantConfig
 

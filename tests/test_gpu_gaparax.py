@@ -246,7 +246,7 @@ def attention_kernels(q, k, v, wq, wk, form_args, scale, dtype, dev, portions, m
         seqops.rope_norm_store(proj, 0, H * d, H * d + G * d, H, G, d, e, None, 0, None, EPS, True, b, kp, vp, q_norm_w=wq.float().to(dev),
                                k_norm_w=wk.float().to(dev))
         acc, ml, ns = seqops.window_attention(proj, 0, kp, vp, b, scale, 0, H, G, d, e, all_kv=False, mfma=mfma, n_splits=n_splits, form=form)
-        out.append(seqops.head_mix_gate(acc, ml, ns, None, None, None, 0, b, H, G, e, torch.float32, plain_sum=True))
+        out.append(seqops.head_mix_gate(acc, ml, ns, None, None, None, 0, b, H, G, e, torch.float32, plain_sum=bool(form_args.get("sigmoid"))))
         at += n
     assert at == T
     return torch.cat(out).reshape(T, H, e)
@@ -322,6 +322,27 @@ def test_sigmoid_attention_bias_rows_cap_and_head_factor_show(dev, dtype):
         for mfma in (True, False):
             got = attention_kernels(q, k, v, wq, wk, args, 0.25, dtype, dev, [120, 1, 1, 1, 77], mfma=mfma, shuffle_pages=True)
             assert_close(got.reshape(T, -1), ref.reshape(T, -1), dtype, (rows, far, chunk, mfma))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_score_form_with_a_softmax(dev, dtype):
+    """the same score form (factor per head, cap, distance bias, chunks) under a softmax instead of sigmoids: the splits are merged with
+    their maxima and sums"""
+    from zhilight_amd import mixers
+    T, H, G, d, e, chunk, cap, far, scale = 200, 4, 2, 24, 16, 70, 3.0, 40, 0.3
+    g = torch.Generator().manual_seed(11)
+    q, k, v = bf(torch.randn(T, H, d, generator=g)), bf(torch.randn(T, G, d, generator=g)), bf(torch.randn(T, G, e, generator=g))
+    wq, wk = bf(1.0 + 0.2 * torch.randn(d, generator=g)), bf(1.0 + 0.2 * torch.randn(d, generator=g))
+    temp, table = bf(torch.tensor([0.5, 2.0, 1.0, 4.0])), bf(torch.randn(10, H, generator=g))
+    qn, kn, bias, vis = O.rms_norm(q, wq, EPS), O.rms_norm(k, wk, EPS), O.distance_bias(T, table, far), O.chunk_visible(T, chunk)
+    ref = torch.zeros(T, H, e, dtype=F64)
+    for a in range(H):
+        sc = cap * torch.tanh((qn[:, a] @ kn[:, a // 2].T) * scale * temp[a] / cap) + bias[a]
+        ref[:, a] = torch.softmax(sc.masked_fill(~vis, -math.inf), -1) @ v[:, a // 2]
+    args = dict(head_scale=temp, softcap=cap, bias=mixers.distance_bias_table(table.float(), far, chunk, "cpu"), chunk=chunk)
+    for mfma, splits in ((True, None), (False, 2)):
+        got = attention_kernels(q, k, v, wq, wk, args, scale, dtype, dev, [130, 1, 1, 68], mfma=mfma, n_splits=splits)
+        assert_close(got.reshape(T, -1), ref.reshape(T, -1), dtype, mfma)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

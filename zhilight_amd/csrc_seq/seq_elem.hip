@@ -189,12 +189,17 @@ template <int DT>
 __global__ __launch_bounds__(kT) void k_streams_norm(const StreamsP p) {
     extern __shared__ float u[];
     __shared__ float red[16];
+    float rc[kMaxStreams];
+#pragma unroll
+    for (int s = 0; s < kMaxStreams; ++s) rc[s] = s < p.n ? (p.read_coef ? p.read_coef[s] : 1.0f) : 0.f;
     const size_t row = p.rows ? (size_t)p.rows[blockIdx.x] : (size_t)blockIdx.x;
     const float* x = p.src + row * p.src_tok;
     float ss = 0.f;
     for (int i = threadIdx.x; i < p.width; i += kT) {
         float a = 0.f;
-        for (int s = 0; s < p.n; ++s) a = fmaf(p.read_coef ? p.read_coef[s] : 1.0f, x[(size_t)s * p.src_stream + i], a);
+#pragma unroll
+        for (int s = 0; s < kMaxStreams; ++s)
+            if (s < p.n) a = fmaf(rc[s], x[(size_t)s * p.src_stream + i], a);
         u[i] = a;
         ss = fmaf(a, a, ss);
     }
@@ -202,34 +207,71 @@ __global__ __launch_bounds__(kT) void k_streams_norm(const StreamsP p) {
     for (int i = threadIdx.x; i < p.width; i += kT) SeqT<DT>::st(p.h, (size_t)blockIdx.x * p.width + i, u[i] * f * (p.w[i] + p.shift));
 }
 
-// x_t <- sum_s mix[s][t] x_s + out_coef[t] * y * sigmoid(gate + bias), all streams from the old ones (a thread holds its element of every
-// stream in registers before it writes); with read_coef also the NEXT sub-layer's input, the normed weighted sum of the new streams
-template <int DT>
+// V consecutive fp32 numbers (V = 4: one 16-byte access)
+template <int V> struct VecF;
+template <> struct VecF<1> {
+    static __device__ __forceinline__ void ld(const float* p, float* v) { v[0] = *p; }
+    static __device__ __forceinline__ void st(float* p, const float* v) { *p = v[0]; }
+};
+template <> struct VecF<4> {
+    static __device__ __forceinline__ void ld(const float* p, float* v) {
+        const float4 a = *reinterpret_cast<const float4*>(p);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    }
+    static __device__ __forceinline__ void st(float* p, const float* v) { *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]); }
+};
+
+// x_t <- sum_s mix[s][t] x_s + out_coef[t] * y * sigmoid(gate + bias), all streams from the old ones (a thread holds its elements of every
+// stream in registers before it writes); with read_coef also the NEXT sub-layer's input, the normed weighted sum of the new streams.
+// N streams (the coefficients sit in registers, every loop unrolled), V elements per thread and access.
+template <int DT, int N, int V>
 __global__ __launch_bounds__(kT) void k_streams_update(const StreamsP p) {
     extern __shared__ float u[];
     __shared__ float red[16];
+    float cm[N][N], co[N], cr[N];
+#pragma unroll
+    for (int s = 0; s < N; ++s) {
+#pragma unroll
+        for (int d = 0; d < N; ++d) cm[s][d] = p.mix[s * N + d];
+        co[s] = p.out_coef[s];
+        cr[s] = p.read_coef ? p.read_coef[s] : 0.f;
+    }
     const size_t t = blockIdx.x;
     const float* x = p.src + t * p.src_tok;
-    float* o = p.dst + t * (size_t)p.n * p.width;
+    float* o = p.dst + t * (size_t)N * p.width;
     float ss = 0.f;
-    for (int i = threadIdx.x; i < p.width; i += kT) {
-        float old[kMaxStreams];
+    for (int i = threadIdx.x * V; i < p.width; i += kT * V) {
+        float old[N][V], yv[V];
 #pragma unroll
-        for (int s = 0; s < kMaxStreams; ++s) old[s] = s < p.n ? x[(size_t)s * p.src_stream + i] : 0.f;
-        float yv = p.y[t * p.width + i];
-        if (p.gate) yv *= seq_sigmoid(p.gate[t * p.ldg + p.g_col0 + i] + (p.gate_bias ? p.gate_bias[i] : 0.f));
-        float a = 0.f;
-        for (int d = 0; d < p.n; ++d) {
-            float v = 0.f;
+        for (int s = 0; s < N; ++s) VecF<V>::ld(x + (size_t)s * p.src_stream + i, old[s]);
+        VecF<V>::ld(p.y + t * p.width + i, yv);
+        if (p.gate) {
+            float g[V], gb[V];
+            VecF<V>::ld(p.gate + t * p.ldg + p.g_col0 + i, g);
 #pragma unroll
-            for (int s = 0; s < kMaxStreams; ++s)
-                if (s < p.n) v = fmaf(p.mix[s * p.n + d], old[s], v);
-            v = fmaf(p.out_coef[d], yv, v);
-            o[(size_t)d * p.width + i] = v;
-            if (p.read_coef) a = fmaf(p.read_coef[d], v, a);
+            for (int e = 0; e < V; ++e) gb[e] = 0.f;
+            if (p.gate_bias) VecF<V>::ld(p.gate_bias + i, gb);
+#pragma unroll
+            for (int e = 0; e < V; ++e) yv[e] *= seq_sigmoid(g[e] + gb[e]);
         }
-        u[i] = a;
-        ss = fmaf(a, a, ss);
+        float a[V];
+#pragma unroll
+        for (int e = 0; e < V; ++e) a[e] = 0.f;
+#pragma unroll
+        for (int d = 0; d < N; ++d) {
+            float v[V];
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                float acc = 0.f;
+#pragma unroll
+                for (int s = 0; s < N; ++s) acc = fmaf(cm[s][d], old[s][e], acc);
+                v[e] = fmaf(co[d], yv[e], acc);
+                a[e] = fmaf(cr[d], v[e], a[e]);
+            }
+            VecF<V>::st(o + (size_t)d * p.width + i, v);
+        }
+#pragma unroll
+        for (int e = 0; e < V; ++e) { u[i + e] = a[e]; ss = fmaf(a[e], a[e], ss); }
     }
     if (!p.read_coef) return;
     const float f = 1.0f / sqrtf(zl_block_sum(ss, red) / (float)p.width + p.eps);
@@ -363,9 +405,23 @@ extern "C" int zls_streams_update(const float* src, int64_t src_tok, int64_t src
     p.src = src; p.src_tok = src_tok; p.src_stream = src_stream; p.dst = dst; p.n = (int)n; p.width = (int)width; p.y = y; p.gate = gate;
     p.ldg = ldg; p.g_col0 = (int)g_col0; p.gate_bias = gate_bias; p.mix = mix; p.out_coef = out_coef; p.read_coef = read_coef; p.w = w;
     p.shift = shift; p.eps = eps; p.h = h;
-#define CALL(DT) hipLaunchKernelGGL((k_streams_update<DT>), dim3((unsigned)n_tok), dim3(kT), (size_t)width * sizeof(float), (hipStream_t)s, p);
+    // 16-byte accesses when every row that is read or written starts on a 16-byte boundary
+    auto al = [](const void* q) { return ((uintptr_t)q & 15) == 0; };
+    const bool vec = width % 4 == 0 && src_tok % 4 == 0 && src_stream % 4 == 0 && al(src) && al(dst) && al(y) &&
+                     (!gate || (ldg % 4 == 0 && g_col0 % 4 == 0 && al(gate))) && (!gate_bias || al(gate_bias));
+    const dim3 grid((unsigned)n_tok);
+    const size_t lds = (size_t)width * sizeof(float);
+#define GO(DT, N)                                                                                          \
+    if (vec) hipLaunchKernelGGL((k_streams_update<DT, N, 4>), grid, dim3(kT), lds, (hipStream_t)s, p);     \
+    else hipLaunchKernelGGL((k_streams_update<DT, N, 1>), grid, dim3(kT), lds, (hipStream_t)s, p);
+#define CALL(DT)                                                                                           \
+    switch (n) {                                                                                           \
+        case 1: GO(DT, 1) break; case 2: GO(DT, 2) break; case 3: GO(DT, 3) break; case 4: GO(DT, 4) break; \
+        case 5: GO(DT, 5) break; case 6: GO(DT, 6) break; case 7: GO(DT, 7) break; default: GO(DT, 8) break; \
+    }
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
+#undef GO
     return zl_launch_status();
 }
 

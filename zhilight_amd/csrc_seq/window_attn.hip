@@ -298,7 +298,8 @@ __device__ __forceinline__ float fast_sigmoid(float x) {
 }
 __device__ __forceinline__ float fast_tanh(float x) { return 2.0f * fast_sigmoid(2.0f * x) - 1.0f; }
 
-template <int KS, int FORM>             // 32-coordinate steps of the head size: dim <= 32 KS; FORM 1: the general score form of AttnP
+template <int KS, int FORM>             // 32-coordinate steps of the head size: dim <= 32 KS; FORM 1: the general score form of AttnP with a
+                                        // softmax, 2: with sigmoid weights (no maximum, no correction of the sums, no normaliser)
 __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, const zls_batch_t b) {
     __shared__ uint4 pfrag[2][4][2][2][64];                              // [buffer][query block][key half][hi, lo][lane]
     __shared__ float corr_s[2][64], l_s[64], m_s[64];
@@ -320,6 +321,8 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
     const float qscale = (FORM && p.head_scale) ? p.scale * p.head_scale[g] : p.scale;
     const int chunk0 = (FORM && p.chunk > 0) ? pq / p.chunk * p.chunk : 0;          // the first position of the query's chunk
     const float off = (FORM && p.offset) ? p.offset[g] : 0.f;
+    const float inv_cap = (FORM && p.softcap > 0.f) ? 1.0f / p.softcap : 0.f;
+    const bool bias_lds = FORM && p.bias && p.bias_rows <= kBiasLds;     // (uniform: the whole row of the head sits in LDS)
     if (FORM && p.bias) {
         for (int i = tid; i < min(p.bias_rows, kBiasLds); i += 256) bias_s[i] = p.bias[(size_t)g * p.bias_rows + i];
         __syncthreads();
@@ -391,18 +394,21 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
                 vis[kb][r] = qok && j <= pq && (p.window <= 0 || pq - j < p.window || j < p.keep_first) && (!FORM || j >= chunk0);
                 if (FORM && vis[kb][r]) {
                     float sv = st[kb][r];
-                    if (p.softcap > 0.f) sv = p.softcap * fast_tanh(sv * __builtin_amdgcn_rcpf(p.softcap));
-                    if (p.bias) {
+                    if (p.softcap > 0.f) sv = p.softcap * fast_tanh(sv * inv_cap);
+                    if (bias_lds) sv += bias_s[min(pq - j, p.bias_rows - 1)];
+                    else if (p.bias) {
                         const int bi = min(pq - j, p.bias_rows - 1);
                         sv += bi < kBiasLds ? bias_s[bi] : p.bias[(size_t)g * p.bias_rows + bi];
                     }
                     st[kb][r] = sv;
                 }
-                if (vis[kb][r]) cm = fmaxf(cm, st[kb][r]);
+                if (FORM != 2 && vis[kb][r]) cm = fmaxf(cm, st[kb][r]);
             }
-        cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
-        cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
-        const bool sig = FORM && p.sigmoid;
+        constexpr bool sig = FORM == 2;
+        if (!sig) {
+            cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
+            cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
+        }
         const float m_new = sig ? 0.f : fmaxf(m_run, cm);
         // (this kernel serves bf16 only: the hardware's exp2 is accurate to 1 ulp of the fp32 result, far inside what the bf16 keys leave)
         constexpr float kLog2e = 1.4426950408889634f;
@@ -415,8 +421,10 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
                 pw[kb][r] = !vis[kb][r] ? 0.f : sig ? fast_sigmoid(st[kb][r] + off) : __builtin_amdgcn_exp2f((st[kb][r] - m_new) * kLog2e);
                 psum += pw[kb][r];
             }
-        psum += __shfl_xor(psum, 16, 64);
-        psum += __shfl_xor(psum, 32, 64);
+        if (!sig) {
+            psum += __shfl_xor(psum, 16, 64);
+            psum += __shfl_xor(psum, 32, 64);
+        }
         l_run = sig ? 1.0f : l_run * corr + psum;                         // (sigmoid weights: nothing to normalise, ml = (0, 1))
         m_run = m_new;
 #pragma unroll
@@ -428,16 +436,18 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
             pfrag[buf][wave][h2][0][lane] = hi;
             pfrag[buf][wave][h2][1][lane] = lo;
         }
-        if (kq == 0) corr_s[buf][qi] = corr;
+        if (!sig && kq == 0) corr_s[buf][qi] = corr;
         __syncthreads();
         // ---- O^T += V^T P^T for this wave's output blocks and all four query blocks
-        float cq[4];
+        if (!sig) {
+            float cq[4];
 #pragma unroll
-        for (int qb = 0; qb < 4; ++qb) cq[qb] = corr_s[buf][16 * qb + nrow];
+            for (int qb = 0; qb < 4; ++qb) cq[qb] = corr_s[buf][16 * qb + nrow];
 #pragma unroll
-        for (int i = 0; i < kItems; ++i)
+            for (int i = 0; i < kItems; ++i)
 #pragma unroll
-            for (int qb = 0; qb < 4; ++qb) acc[i][qb] *= cq[qb];
+                for (int qb = 0; qb < 4; ++qb) acc[i][qb] *= cq[qb];
+        }
 #pragma unroll
         for (int h2 = 0; h2 < 2; ++h2) {
             uint4 vf[kItems];
@@ -691,7 +701,8 @@ extern "C" int zls_window_attention_prompt(const float* q, int64_t ldq, int64_t 
     hipStream_t hs = (hipStream_t)s;
     const int ks = (int)((dim + 31) / 32);
 #define PROMPT(KS)                                                                                      \
-    if (form) hipLaunchKernelGGL((k_window_attention_mfma<KS, 1>), grid, dim3(256), 0, hs, p, *b);      \
+    if (form && form->sigmoid) hipLaunchKernelGGL((k_window_attention_mfma<KS, 2>), grid, dim3(256), 0, hs, p, *b); \
+    else if (form) hipLaunchKernelGGL((k_window_attention_mfma<KS, 1>), grid, dim3(256), 0, hs, p, *b); \
     else hipLaunchKernelGGL((k_window_attention_mfma<KS, 0>), grid, dim3(256), 0, hs, p, *b)
     if (ks <= 1) { PROMPT(1); }
     else if (ks <= 2) { PROMPT(2); }
