@@ -278,17 +278,21 @@ __global__ __launch_bounds__(kT) void k_streams_update(const StreamsP p) {
     for (int i = threadIdx.x; i < p.width; i += kT) SeqT<DT>::st(p.h, t * p.width + i, u[i] * f * (p.w[i] + p.shift));
 }
 
-// out = act(z): kind 0 relu(z)^2, 1 gelu_tanh(z), 2 silu(z)
-template <int DT>
+// out = act(z): kind 0 relu(z)^2, 1 gelu_tanh(z), 2 silu(z); V consecutive elements of a row per thread
+template <int DT, int V>
 __global__ __launch_bounds__(kT) void k_unary_act(const float* __restrict__ z, int64_t ldz, int64_t rows, int64_t cols, int kind, void* __restrict__ out) {
-    const int64_t e = (int64_t)blockIdx.x * kT + threadIdx.x;
+    const int64_t e = ((int64_t)blockIdx.x * kT + threadIdx.x) * V;
     if (e >= rows * cols) return;
-    const float v = z[(e / cols) * ldz + e % cols];
-    float r;
-    if (kind == 0) { const float m = fmaxf(v, 0.f); r = m * m; }
-    else if (kind == 1) r = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
-    else r = seq_silu(v);
-    SeqT<DT>::st(out, (size_t)e, r);
+    float v[V];
+    VecF<V>::ld(z + (e / cols) * ldz + e % cols, v);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+        float r;
+        if (kind == 0) { const float m = fmaxf(v[i], 0.f); r = m * m; }
+        else if (kind == 1) r = 0.5f * v[i] * (1.0f + tanhf(0.7978845608028654f * (v[i] + 0.044715f * v[i] * v[i] * v[i])));
+        else r = seq_silu(v[i]);
+        SeqT<DT>::st(out, (size_t)e + i, r);
+    }
 }
 
 }  // namespace
@@ -429,7 +433,11 @@ extern "C" int zls_unary_act(const float* z, int64_t ldz, int64_t rows, int64_t 
     ZL_CHECK_ARG(z && out && rows > 0 && cols > 0 && ldz >= cols && kind >= 0 && kind <= 2, ZL_EINVAL);
     const int64_t n = rows * cols;
     ZL_CHECK_ARG(n < (1LL << 40), ZL_ELIMIT);
-#define CALL(DT) hipLaunchKernelGGL((k_unary_act<DT>), dim3((unsigned)((n + kT - 1) / kT)), dim3(kT), 0, (hipStream_t)s, z, ldz, rows, cols, kind, out);
+    const bool vec = cols % 4 == 0 && ldz % 4 == 0 && ((uintptr_t)z & 15) == 0;
+    hipStream_t hs = (hipStream_t)s;
+#define CALL(DT)                                                                                                                     \
+    if (vec) hipLaunchKernelGGL((k_unary_act<DT, 4>), dim3((unsigned)((n / 4 + kT - 1) / kT)), dim3(kT), 0, hs, z, ldz, rows, cols, kind, out); \
+    else hipLaunchKernelGGL((k_unary_act<DT, 1>), dim3((unsigned)((n + kT - 1) / kT)), dim3(kT), 0, hs, z, ldz, rows, cols, kind, out);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
     return zl_launch_status();
