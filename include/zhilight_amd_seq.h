@@ -276,8 +276,9 @@ int zls_lowrank_decay(const float* proj, int64_t ld, int64_t u_col0, int64_t low
  * correction (nullable); the outputs form `groups` equal groups of neighbours, a group's score is the sum of its `group_top` largest choice
  * scores (1: its largest), only outputs of the `keep` best groups can be chosen (groups <= 1: all) -- the others count as minus
  * infinity; the `top` largest choice scores are chosen (ties: the lower index).  ids int32 (n_tok, top), weights fp32 (n_tok, top) = s of
- * the chosen (divided by their sum + renorm_eps when renorm != 0), times weight_scale.  n_out <= 1024, n_out % groups == 0. */
-int zls_moe_route(const float* logits, int64_t n_tok, int64_t n_out, const float* correction, int64_t groups, int64_t keep, int64_t top,
+ * the chosen (divided by their sum + renorm_eps when renorm != 0), times weight_scale.  n_out <= 1024, n_out % groups == 0.  A token's
+ * logits are the first n_out numbers of its row of ld >= n_out numbers. */
+int zls_moe_route(const float* logits, int64_t ld, int64_t n_tok, int64_t n_out, const float* correction, int64_t groups, int64_t keep, int64_t top,
                   int renorm, int score_kind, int64_t group_top, float renorm_eps, float weight_scale, int32_t* ids, float* weights,
                   zl_stream_t s);
 /* Sort the n_slots = n_tok * top (token, choice) pairs by expert: pairs whose id is >= n_experts (identity outputs) are left out.

@@ -22,12 +22,12 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {          // larg
     }
 }
 
-__global__ __launch_bounds__(64) void k_moe_route(const float* __restrict__ logits, int n_out, const float* __restrict__ correction, int groups,
+__global__ __launch_bounds__(64) void k_moe_route(const float* __restrict__ logits, int64_t ld, int n_out, const float* __restrict__ correction, int groups,
                                                   int keep, int top, int renorm, int score_kind, int group_top, float renorm_eps,
                                                   float weight_scale, int32_t* __restrict__ ids, float* __restrict__ weights) {
     __shared__ float prob[1024], choice[1024], gscore[1024];
     const int t = blockIdx.x, lane = threadIdx.x;
-    const float* z = logits + (size_t)t * n_out;
+    const float* z = logits + (size_t)t * ld;                          // (the router's columns may lead wider rows)
     float mx = -INFINITY;
     for (int i = lane; i < n_out; i += 64) mx = fmaxf(mx, z[i]);
     mx = zl_wave_max(mx);
@@ -206,15 +206,15 @@ __global__ __launch_bounds__(256) void k_moe_combine(const float* __restrict__ y
 
 }  // namespace
 
-extern "C" int zls_moe_route(const float* logits, int64_t n_tok, int64_t n_out, const float* correction, int64_t groups, int64_t keep, int64_t top,
+extern "C" int zls_moe_route(const float* logits, int64_t ld, int64_t n_tok, int64_t n_out, const float* correction, int64_t groups, int64_t keep, int64_t top,
                              int renorm, int score_kind, int64_t group_top, float renorm_eps, float weight_scale, int32_t* ids, float* weights,
                              zl_stream_t s) {
-    ZL_CHECK_ARG(logits && ids && weights && n_tok > 0 && n_out > 0 && top > 0, ZL_EINVAL);
+    ZL_CHECK_ARG(logits && ids && weights && n_tok > 0 && n_out > 0 && top > 0 && ld >= n_out, ZL_EINVAL);
     ZL_CHECK_ARG(n_out <= 1024 && top <= n_out, ZL_ELIMIT);
     if (groups < 1) groups = 1;
     ZL_CHECK_ARG(n_out % groups == 0 && keep >= 1 && keep <= groups && top <= keep * (n_out / groups), ZL_ESHAPE);
     ZL_CHECK_ARG((score_kind == 0 || score_kind == 1) && group_top >= 1, ZL_EINVAL);
-    hipLaunchKernelGGL(k_moe_route, dim3((unsigned)n_tok), dim3(64), 0, (hipStream_t)s, logits, (int)n_out, correction, (int)groups, (int)keep,
+    hipLaunchKernelGGL(k_moe_route, dim3((unsigned)n_tok), dim3(64), 0, (hipStream_t)s, logits, ld, (int)n_out, correction, (int)groups, (int)keep,
                        (int)top, renorm, score_kind, (int)group_top, renorm_eps, weight_scale, ids, weights);
     return zl_launch_status();
 }

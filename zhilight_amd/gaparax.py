@@ -18,9 +18,9 @@ Tensors: embed, head, final.norm, l<i>.norm1 / norm2, l<i>.hc1 / hc2 .in / .out 
 the mixer classes in mixers.py).
 
 The model runs RAGGED steps like the other models of the engine: every launch covers all tokens of a step; cached rows live in paged
-planes of the engine's CacheManager.  The gate's projection rides in the sub-layer's own input product where that is one product (the
-mixers, the dense feed-forward), and one launch between two products writes the streams AND the next sub-layer's normed input, so a layer
-is: product, mixer kernels, product, streams update, feed-forward launches, streams update.
+planes of the engine's CacheManager.  The gate's projection rides in the sub-layer's own first product (the mixers' input projection,
+the dense feed-forward's up projection, the experts' router), and one launch between two products writes the streams AND the next
+sub-layer's normed input, so a layer is: product, mixer kernels, product, streams update, feed-forward launches, streams update.
 """
 from dataclasses import dataclass, field
 from typing import List, Optional
@@ -136,6 +136,7 @@ class StreamPort:
         self.fused = hasattr(sub, "attach_side")
         if self.fused:
             sub.attach_side(self.gate_w)
+            self.gate_w = None                         # (the rows live in the sub-layer's matrix now)
 
     def gate_of(self, sub, h):
         """(fp32 tensor, first column) of W_rg h"""

@@ -651,7 +651,7 @@ class MLSTMMixer:
         return seqops.gemm_nt(a, self.w_o)
 
 
-class RoutedExpertsFF:
+class RoutedExpertsFF(SideRows):
     """Mixture of gated feed-forward experts, down(silu(gate h) * (up h)), without biases.  The router gives one logit per expert and per
     IDENTITY output (the last `identity` of its outputs: their "expert" returns h itself); probabilities = softmax over all outputs; an
     output is chosen by probability + `correction`, within the `keep` best of `groups` equal groups of neighbouring outputs (a group scores
@@ -660,6 +660,7 @@ class RoutedExpertsFF:
     Tensors under `prefix`: router (experts + identity, width), correction (experts + identity), e<j>.gate / e<j>.up (ff, width),
     e<j>.down (width, ff).  Gate and up rows of all experts are stacked in blocks of 16 (16 gate rows, their 16 up rows), so that the grouped
     product's epilogue finishes the activation."""
+    _side_matrix = "w_router"
 
     def __init__(self, width, ff, experts, top, identity=0, groups=1, keep=1, correction=True, renorm=False, score="softmax", group_top=1,
                  renorm_eps=0.0, act="silu", act_alpha=1.0, limit=0.0, weight_scale=1.0):
@@ -708,12 +709,14 @@ class RoutedExpertsFF:
         return self
 
     def weight_bytes(self):
-        return sum(t.numel() * t.element_size() for t in (self.w_router, self.w_gu, self.w_down))
+        return sum(t.numel() * t.element_size() for t in (self.w_router, self.w_gu, self.w_down))       # (w_router: with attached side rows)
 
     def forward(self, h):
-        logits = seqops.gemm_nt(h, self.w_router)                                 # fp32 sums of the products
+        logits = seqops.gemm_nt(h, self.w_router)                                 # fp32 sums of the products [router | side rows]
+        self.side = (logits, self.side_col0)
         ids, weights = seqops.moe_route(logits, self.correction, self.groups, self.keep, self.top, self.renorm, score=self.score,
-                                        group_top=self.group_top, renorm_eps=self.renorm_eps, weight_scale=self.weight_scale)
+                                        group_top=self.group_top, renorm_eps=self.renorm_eps, weight_scale=self.weight_scale,
+                                        n_out=self.experts + self.identity)
         sorted_tok, slot_pos, tiles, max_tiles, sorted_exp, tm = seqops.moe_align(ids, self.experts, self.tile_m)
         n_slots = ids.numel()
         few = sorted_exp if n_slots <= self.few_rows else None                    # decode steps: weight rows streamed per (row, column)

@@ -660,17 +660,21 @@ MOE_TILE = 64           # rows of an expert's tile in the grouped products; 128 
 MOE_BIG_SHARE = 256
 
 
-def moe_route(logits, correction, groups, keep, top, renorm=False, score="softmax", group_top=1, renorm_eps=0.0, weight_scale=1.0):
+def moe_route(logits, correction, groups, keep, top, renorm=False, score="softmax", group_top=1, renorm_eps=0.0, weight_scale=1.0, n_out=None):
+    """n_out: the router's outputs are the leading n_out columns of wider rows (None: all columns)"""
     _cuda(logits, correction)
     _f32(logits, correction)
-    n_tok, n_out = logits.shape
+    n_tok = logits.shape[0]
+    n_out = logits.shape[1] if n_out is None else int(n_out)
+    if n_out > logits.shape[1]:
+        raise ZLError("moe_route: more router outputs than columns")
     if correction is not None and correction.numel() != n_out:
         raise ZLError("moe_route: one correction per router output")
     ids = torch.empty((n_tok, top), dtype=torch.int32, device=logits.device)
     weights = torch.empty((n_tok, top), dtype=torch.float32, device=logits.device)
     if score not in ("softmax", "sigmoid"):
         raise ZLError("moe_route: scores are softmax or sigmoid")
-    check(lib().zls_moe_route(_p(logits), _i(n_tok), _i(n_out), _p(correction), _i(groups), _i(keep), _i(top), C.c_int(int(renorm)),
+    check(lib().zls_moe_route(_p(logits), _i(logits.stride(0)), _i(n_tok), _i(n_out), _p(correction), _i(groups), _i(keep), _i(top), C.c_int(int(renorm)),
                               C.c_int(1 if score == "sigmoid" else 0), _i(group_top), _f(renorm_eps), _f(weight_scale), _p(ids), _p(weights), _stream()),
           "moe_route")
     return ids, weights
