@@ -664,3 +664,32 @@ def test_greedy_generation_through_the_scheduler(dev):
             if float(top2[0] - top2[1]) > 1e-3:                                 # (a tie within rounding may go either way)
                 assert int(torch.argmax(logits[-1])) == tok
             seq.append(tok)
+
+
+def test_trace_replayer_on_a_model_folder(dev, tmp_path, capsys):
+    """a folder with config.json and model.safetensors through the registry's loader and the trace replayer: two requests in mixed steps
+    (a portion beside single tokens), one leaves and its pages are taken again; the written logits are the restatement's"""
+    import io
+    import json
+    from safetensors.torch import save_file
+    from zhilight_amd import trace
+    cfg = cfg_a()
+    sd = O.random_weights(cfg, 33, fixed_choice=True)
+    folder, out = tmp_path / "model", tmp_path / "out"
+    folder.mkdir()
+    (folder / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.contiguous() for k, v in sd.items()}, str(folder / "model.safetensors"))
+    a, b, c = tokens_of(cfg, 90, 1), tokens_of(cfg, 70, 2), tokens_of(cfg, 100, 3)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:60], "want": [0, 59]}, {"id": "b", "tokens": b[:2], "want": [1]}], "end": []},
+             {"step": 1, "entries": [{"id": "b", "tokens": b[2:70], "want": [67]}, {"id": "a", "tokens": a[60:61], "want": [0]}], "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[61:90], "want": []}], "end": []},
+             {"step": 3, "entries": [{"id": "c", "tokens": c, "want": [99]}, {"id": "a", "tokens": [a[0]], "want": [0]}], "end": ["a", "c"]}]
+    stream = io.StringIO("".join(json.dumps(s) + "\n" for s in steps))
+    assert trace.replay(str(folder), "float32", str(out), max_tokens=256, max_seqs=2, stream=stream, device=str(dev)) == 0
+    assert [l for l in capsys.readouterr().out.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2", "done 3"]
+    la, lb, lc = O.model(a + [a[0]], sd, cfg), O.model(b, sd, cfg), O.model(c, sd, cfg)
+    want = {0: torch.stack([la[0], la[59], lb[1]]), 1: torch.stack([lb[69], la[60]]), 3: torch.stack([lc[99], la[90]])}
+    assert not (out / "2.f32").exists()
+    for n, ref in want.items():
+        got = torch.from_numpy(np.fromfile(str(out / f"{n}.f32"), dtype="<f4").reshape(ref.shape[0], cfg["vocab"]))
+        assert_close(got, ref, torch.float32, f"step {n}")

@@ -323,8 +323,23 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
     const float off = (FORM && p.offset) ? p.offset[g] : 0.f;
     const float inv_cap = (FORM && p.softcap > 0.f) ? 1.0f / p.softcap : 0.f;
     const bool bias_lds = FORM && p.bias && p.bias_rows <= kBiasLds;     // (uniform: the whole row of the head sits in LDS)
+    // Sigmoid weights (FORM 2) in as few instructions per score as the form allows.  With r = 1 / (1 + 2^(k1 s)), k1 = -2 log2(e) / cap,
+    // the capped score is 2 cap r - cap, so the weight is 1 / (1 + 2^z) with z = A r + b[distance]: A = -2 cap log2(e) and
+    // b = -log2(e) (bias + offset - cap), which is what the LDS row holds here; without a cap r = s and A = -log2(e).
+    constexpr float kL2e = 1.4426950408889634f;
+    const bool has_cap = FORM && p.softcap > 0.f;
+    const float sg_k1 = has_cap ? -2.0f * kL2e * inv_cap : 0.f, sg_a = has_cap ? -2.0f * kL2e * p.softcap : -kL2e;
+    const float sg_c0 = -kL2e * (off - (has_cap ? p.softcap : 0.f));
+    // a key at distance dq = pq - j is visible iff 0 <= dq <= dmax (chunk and window in one unsigned comparison); kept first keys
+    // need the general test
+    const bool fast_vis = FORM == 2 && p.keep_first == 0;
+    const int pq_eff = qok ? pq : -(1 << 30);
+    const unsigned dmax = qok ? (unsigned)min(pq - chunk0, p.window > 0 ? p.window - 1 : pq) : 0u;
     if (FORM && p.bias) {
-        for (int i = tid; i < min(p.bias_rows, kBiasLds); i += 256) bias_s[i] = p.bias[(size_t)g * p.bias_rows + i];
+        for (int i = tid; i < min(p.bias_rows, kBiasLds); i += 256) {
+            const float bv = p.bias[(size_t)g * p.bias_rows + i];
+            bias_s[i] = FORM == 2 ? fmaf(-kL2e, bv, sg_c0) : bv;
+        }
         __syncthreads();
     }
     uint4 qh[KS], ql[KS];
@@ -386,8 +401,24 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
         // st[kb][r]: key pg * 64 + 16 kb + 4 kq + r, query nrow
         float cm = -INFINITY;
         bool vis[4][4];
+        float pw[4][4], psum = 0.f;
+        if (FORM == 2) {
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb)
+            for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int j = pg * 64 + 16 * kb + 4 * kq + r;
+                    const int dq = pq_eff - j;
+                    const bool v = fast_vis ? (unsigned)dq <= dmax
+                                            : (qok && j <= pq && (p.window <= 0 || pq - j < p.window || j < p.keep_first) && j >= chunk0);
+                    const unsigned bi = min((unsigned)dq, (unsigned)(p.bias_rows - 1));
+                    const float rr = has_cap ? __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(sg_k1 * st[kb][r])) : st[kb][r];
+                    const float bb = bias_lds ? bias_s[bi] : (p.bias ? fmaf(-kL2e, p.bias[(size_t)g * p.bias_rows + bi], sg_c0) : sg_c0);
+                    pw[kb][r] = v ? __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(fmaf(sg_a, rr, bb))) : 0.f;
+                }
+        }
+#pragma unroll
+        for (int kb = 0; FORM != 2 && kb < 4; ++kb)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int j = pg * 64 + 16 * kb + 4 * kq + r;
@@ -413,12 +444,11 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
         // (this kernel serves bf16 only: the hardware's exp2 is accurate to 1 ulp of the fp32 result, far inside what the bf16 keys leave)
         constexpr float kLog2e = 1.4426950408889634f;
         const float corr = (sig || m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f((m_run - m_new) * kLog2e);
-        float pw[4][4], psum = 0.f;
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb)
+        for (int kb = 0; !sig && kb < 4; ++kb)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                pw[kb][r] = !vis[kb][r] ? 0.f : sig ? fast_sigmoid(st[kb][r] + off) : __builtin_amdgcn_exp2f((st[kb][r] - m_new) * kLog2e);
+                pw[kb][r] = !vis[kb][r] ? 0.f : __builtin_amdgcn_exp2f((st[kb][r] - m_new) * kLog2e);
                 psum += pw[kb][r];
             }
         if (!sig) {

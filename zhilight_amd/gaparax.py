@@ -74,7 +74,7 @@ class GaparaxConfig:
 
 def _attention(name, width, m, eps):
     mask = m.get("mask") or {}
-    return WindowAttention(name, width, int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"]), float(m["scale"]), 0, 0, 10000.0, 1.0,
+    return WindowAttention(name, width, int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]), int(m["vdim"]), float(m["scale"]), 0, 0, 10000.0, 1.0,
                            eps, qk_norm=True, rotate_values=False, talk=False, gate=True, norm_weight=True, head_scale=True,
                            softcap=float(m.get("softcap") or 0.0), rel_far=int(m["bias_max"]), chunk=int(mask.get("size", 0)), weights="sigmoid")
 
