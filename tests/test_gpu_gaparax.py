@@ -304,17 +304,18 @@ def test_sigmoid_attention_chunk_edges(dev, dtype, chunk):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_sigmoid_attention_bias_rows_cap_and_head_factor_show(dev, dtype):
     """a bias table with large, distinct rows (every bucket edge moves the weights), scores beyond the cap, unequal factors per head; a
-    table that ends before the chunk does (distances beyond it take the last row); no chunks at all"""
+    table that ends before the chunk does (distances beyond it take the last row); no chunks at all; a table of more distances than the
+    matrix-core kernel keeps in LDS"""
     from zhilight_amd import mixers
     T, H, G, d, e = 200, 4, 1, 32, 16
     g = torch.Generator().manual_seed(5)
     q, k, v = bf(torch.randn(T, H, d, generator=g)), bf(torch.randn(T, G, d, generator=g)), bf(torch.randn(T, G, e, generator=g))
     wq, wk = bf(1.0 + 0.3 * torch.randn(d, generator=g)), bf(1.0 + 0.3 * torch.randn(d, generator=g))
     temp, offset = bf(torch.tensor([0.5, 3.0, 1.0, 6.0])), bf(torch.tensor([-2.0, -3.0, -1.0, -4.0]))
-    for rows, far, chunk, cap in ((16, 40, 150, 2.0), (6, 20, 0, 3.0), (12, 300, 90, 0.0)):
+    for rows, far, chunk, cap in ((16, 40, 150, 2.0), (6, 20, 0, 3.0), (12, 300, 90, 0.0), (10, 3000, 0, 3.0)):
         table = bf(torch.linspace(-3.0, 3.0, rows)[:, None] * torch.tensor([1.0, -1.0, 0.5, 2.0])[None, :])
         ref = sigmoid_reference(q, k, v, wq, wk, 0.25, temp, cap, table, far, chunk, offset)
-        assert rel(sigmoid_reference(q, k, v, wq, wk, 0.25, temp, cap, table, 2 * far, chunk, offset), ref) > 0.02       # the buckets show
+        assert far > 1000 or rel(sigmoid_reference(q, k, v, wq, wk, 0.25, temp, cap, table, 2 * far, chunk, offset), ref) > 0.02   # the buckets show
         assert rel(sigmoid_reference(q, k, v, wq, wk, 0.25, temp, 0.0 if cap else 1.0, table, far, chunk, offset), ref) > 0.02   # the cap shows
         assert rel(sigmoid_reference(q, k, v, wq, wk, 0.25, torch.ones(H, dtype=F64), cap, table, far, chunk, offset), ref) > 0.02
         bias = mixers.distance_bias_table(table.float(), far, chunk, "cpu")
@@ -329,20 +330,22 @@ def test_score_form_with_a_softmax(dev, dtype):
     """the same score form (factor per head, cap, distance bias, chunks) under a softmax instead of sigmoids: the splits are merged with
     their maxima and sums"""
     from zhilight_amd import mixers
-    T, H, G, d, e, chunk, cap, far, scale = 200, 4, 2, 24, 16, 70, 3.0, 40, 0.3
+    T, H, G, d, e, cap, scale = 200, 4, 2, 24, 16, 3.0, 0.3
     g = torch.Generator().manual_seed(11)
     q, k, v = bf(torch.randn(T, H, d, generator=g)), bf(torch.randn(T, G, d, generator=g)), bf(torch.randn(T, G, e, generator=g))
     wq, wk = bf(1.0 + 0.2 * torch.randn(d, generator=g)), bf(1.0 + 0.2 * torch.randn(d, generator=g))
     temp, table = bf(torch.tensor([0.5, 2.0, 1.0, 4.0])), bf(torch.randn(10, H, generator=g))
-    qn, kn, bias, vis = O.rms_norm(q, wq, EPS), O.rms_norm(k, wk, EPS), O.distance_bias(T, table, far), O.chunk_visible(T, chunk)
-    ref = torch.zeros(T, H, e, dtype=F64)
-    for a in range(H):
-        sc = cap * torch.tanh((qn[:, a] @ kn[:, a // 2].T) * scale * temp[a] / cap) + bias[a]
-        ref[:, a] = torch.softmax(sc.masked_fill(~vis, -math.inf), -1) @ v[:, a // 2]
-    args = dict(head_scale=temp, softcap=cap, bias=mixers.distance_bias_table(table.float(), far, chunk, "cpu"), chunk=chunk)
-    for mfma, splits in ((True, None), (False, 2)):
-        got = attention_kernels(q, k, v, wq, wk, args, scale, dtype, dev, [130, 1, 1, 68], mfma=mfma, n_splits=splits)
-        assert_close(got.reshape(T, -1), ref.reshape(T, -1), dtype, mfma)
+    qn, kn = O.rms_norm(q, wq, EPS), O.rms_norm(k, wk, EPS)
+    for chunk, far in ((70, 40), (0, 2500)):                                    # (the second table is longer than the kernel's LDS row)
+        bias, vis = O.distance_bias(T, table, far), O.chunk_visible(T, chunk)
+        ref = torch.zeros(T, H, e, dtype=F64)
+        for a in range(H):
+            sc = cap * torch.tanh((qn[:, a] @ kn[:, a // 2].T) * scale * temp[a] / cap) + bias[a]
+            ref[:, a] = torch.softmax(sc.masked_fill(~vis, -math.inf), -1) @ v[:, a // 2]
+        args = dict(head_scale=temp, softcap=cap, bias=mixers.distance_bias_table(table.float(), far, chunk, "cpu"), chunk=chunk)
+        for mfma, splits in ((True, None), (False, 2)):
+            got = attention_kernels(q, k, v, wq, wk, args, scale, dtype, dev, [130, 1, 1, 68], mfma=mfma, n_splits=splits)
+            assert_close(got.reshape(T, -1), ref.reshape(T, -1), dtype, (chunk, mfma))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
